@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void attn_general_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int D, int page,
-    float scale, int window) {
+    float scale, int window, const float* __restrict__ sink) {
   extern __shared__ float smem[];
   const int b = blockIdx.z;
   const int h = blockIdx.y;
@@ -129,7 +129,8 @@ __global__ __launch_bounds__(256) void attn_general_kernel(
     }
   }
   if (my_row) {
-    const float inv = 1.f / l_run;
+    // a sink: one more term of the denominator, exp(sink[h]), with no key and no value behind it
+    const float inv = 1.f / (sink ? l_run + expf(sink[h] - m_run) : l_run);
     T* o = out + (size_t)(q0 + m0 + r) * ((size_t)Hq * D) + (size_t)h * D;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
@@ -141,12 +142,12 @@ template <typename T>
 static int launch_general(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache,
                           int num_pages, const int* block_table, int bt_stride, const int* cu_q,
                           const int* kv_lens, int B, int Hq, int Hkv, int D, int page, float scale,
-                          int window, int max_q_len, hipStream_t stream) {
+                          int window, int max_q_len, const float* sink, hipStream_t stream) {
   const size_t smem = (size_t)(GEN_BM * D + GEN_BN * (D + 1) + GEN_BM * (GEN_BN + 1)) * sizeof(float);
   const dim3 grid((max_q_len + GEN_BM - 1) / GEN_BM, Hq, B);
   hipLaunchKernelGGL(attn_general_kernel<T>, grid, dim3(256), smem, stream, (const T*)q, q_stride, (T*)out,
                      (const T*)k_cache, (const T*)v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens,
-                     Hq, Hkv, D, page, scale, window);
+                     Hq, Hkv, D, page, scale, window, sink);
   return q3_launch_status();
 }
 
@@ -647,7 +648,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, score_scale_t scale_log2,
-    int window, int splits, float* __restrict__ ws_acc, float* __restrict__ ws_ml, DecodePrep prep) {
+    int window, int splits, float* __restrict__ ws_acc, float* __restrict__ ws_ml, DecodePrep prep,
+    const float* __restrict__ sink) {
   const int b = blockIdx.z, g_kv = blockIdx.y, split = blockIdx.x;
   const int G = Hq / Hkv;
   // a step of single tokens (PREP): sequence b's token is row b, and nothing is read to know it
@@ -805,7 +807,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   for (int w = 0; w < 4; ++w) lr += sh_m[w][r] > -INFINITY ? sh_l[w][r] * exp2f(sh_m[w][r] - mr) : 0.f;
   const int token = q0 + r / G, head = g_kv * G + r % G;
   if (splits == 1) {
-    const float inv = 1.f / lr;
+    // a sink joins the denominator once, as 2^(sink log2(e) - maximum): here, or in the merge of the splits
+    const float inv = 1.f / (sink ? lr + exp2f(sink[head] * 1.4426950408889634f - mr) : lr);
     for (int d = dd; d < D; d += 16) {
       float o = sh_acc[0][r][d] + sh_acc[1][r][d] + sh_acc[2][r][d] + sh_acc[3][r][d];
       if (PREP && w5 > 0.f) o += sh_v[d] * w5;
@@ -839,7 +842,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 template <int D>
 __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ cu_q, int Hq, int Hkv, int splits,
-    const float* __restrict__ ws_acc, const float* __restrict__ ws_ml) {
+    const float* __restrict__ ws_acc, const float* __restrict__ ws_ml, const float* __restrict__ sink) {
   __shared__ float sh_w[16][MAX_SPLITS];
   __shared__ float4 sh_part[256];
   const int b = blockIdx.y, g_kv = blockIdx.x;
@@ -875,7 +878,8 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
       if (lane < splits) ml = *reinterpret_cast<const float2*>(ws_ml + ((base + lane) * 16 + r) * 2);
       const float m_all = wave_max(ml.x);
       const float e = ml.x > -INFINITY ? exp2f(ml.x - m_all) : 0.f;
-      const float l_all = wave_sum(ml.y * e);
+      float l_all = wave_sum(ml.y * e);
+      if (sink) l_all += exp2f(sink[g_kv * G + r % G] * 1.4426950408889634f - m_all);
       if (lane < splits) sh_w[r][lane] = l_all > 0.f ? e / l_all : 0.f;   // a row that saw no key at all: zeros
     }
   }
@@ -1055,7 +1059,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, score_scale_t scale_log2,
-    int window, int tokens_per_block, int key_splits, float* __restrict__ part_acc, float* __restrict__ part_ml) {
+    int window, int tokens_per_block, int key_splits, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const float* __restrict__ sink) {
   typedef PrefillSmem<D, TILE> SM;
   constexpr int KB4 = TILE / 16;  // 16-key blocks per tile
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * SM::STAGE];
@@ -1424,6 +1429,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if (grp == 0) *reinterpret_cast<float2*>(part_ml + slot * 2) = make_float2(m_run[qb], l);
       continue;
     }
+    if (sink) l += fast_exp2(sink[row_head[qb]] * 1.4426950408889634f - m_run[qb]);
     const float inv = 1.f / l;
     bf16_t* o = out + (size_t)row_tok[qb] * Hq * D + (size_t)row_head[qb] * D + 4 * grp;
 #pragma unroll
@@ -1446,7 +1452,8 @@ template <int D>
 __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(bf16_t* __restrict__ out,
                                                                  const int* __restrict__ cu_q, int Hq, int Hkv,
                                                                  int key_splits, const float* __restrict__ part_acc,
-                                                                 const float* __restrict__ part_ml) {
+                                                                 const float* __restrict__ part_ml,
+                                                                 const float* __restrict__ sink) {
   const int b = blockIdx.y;
   const int q0 = cu_q[b], q_len = cu_q[b + 1] - q0;
   if (q_len * (Hq / Hkv) <= 16) return;
@@ -1469,6 +1476,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(bf16_t* __restr
       o.x += a.x * w; o.y += a.y * w; o.z += a.z * w; o.w += a.w * w;
       l_all += ml.y * w;
     }
+    if (sink) l_all += fast_exp2(sink[row] * 1.4426950408889634f - m_all);
     const float inv = 1.f / l_all;
     union {
       uint2 u;
@@ -1508,7 +1516,7 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
                        int num_pages, const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens,
                        int B, int total_tokens, int Hq, int Hkv, int page, float scale, int window, int max_q_len,
                        int min_q_len, int splits, float* ws_acc, float* ws_ml, int key_splits, float* prompt_ws,
-                       hipStream_t stream) {
+                       const float* sink, hipStream_t stream) {
   const int G = Hq / Hkv;
   const score_scale_t scale_log2 = make_score_scale(scale);
   if (min_q_len * G <= 16) {
@@ -1516,15 +1524,15 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
       hipLaunchKernelGGL((attn_decode_kernel<D, false, float, true>), dim3(splits, Hkv, B), dim3(256), 0, stream,
                          (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                          num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, splits,
-                         ws_acc, ws_ml, DecodePrep{});
+                         ws_acc, ws_ml, DecodePrep{}, sink);
     else
       hipLaunchKernelGGL((attn_decode_kernel<D, false, float, false>), dim3(splits, Hkv, B), dim3(256), 0, stream,
                          (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                          num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page, scale_log2, window, splits,
-                         ws_acc, ws_ml, DecodePrep{});
+                         ws_acc, ws_ml, DecodePrep{}, sink);
     if (splits > 1)
       hipLaunchKernelGGL(attn_decode_reduce_kernel<D>, dim3(Hkv, B), dim3(256), 0, stream, (bf16_t*)out, cu_q, Hq,
-                         Hkv, splits, ws_acc, ws_ml);
+                         Hkv, splits, ws_acc, ws_ml, sink);
   }
   if (max_q_len * G > 16) {
     const int tokens_per_block = prompt_tokens_per_block(total_tokens, G, Hkv, key_splits);
@@ -1535,10 +1543,10 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
     hipLaunchKernelGGL((attn_prefill_kernel<D, PF_TILE, PF_STAGES>), dim3(Hkv, tiles * key_splits, B), dim3(256), 0,
                        stream, (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_cache,
                        (const bf16_t*)v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page,
-                       scale_log2, window, tokens_per_block, key_splits, part_acc, part_ml);
+                       scale_log2, window, tokens_per_block, key_splits, part_acc, part_ml, sink);
     if (key_splits > 1)
       hipLaunchKernelGGL(attn_prefill_merge_kernel<D>, dim3(max_q_len, B), dim3(256), 0, stream,
-                         (bf16_t*)out, cu_q, Hq, Hkv, key_splits, part_acc, part_ml);
+                         (bf16_t*)out, cu_q, Hq, Hkv, key_splits, part_acc, part_ml, sink);
   }
   return q3_launch_status();
 }
@@ -1553,15 +1561,15 @@ static int launch_decode_prep(const void* qkv, void* out, const void* k_cache, c
     hipLaunchKernelGGL((attn_decode_kernel<D, true, W, true>), dim3(splits, Hkv, B), dim3(256), 0, stream,
                        (const bf16_t*)qkv, (Hq + 2 * Hkv) * D, (bf16_t*)out, (const bf16_t*)k_cache,
                        (const bf16_t*)v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page,
-                       scale_log2, window, splits, ws_acc, ws_ml, prep);
+                       scale_log2, window, splits, ws_acc, ws_ml, prep, (const float*)nullptr);
   else
     hipLaunchKernelGGL((attn_decode_kernel<D, true, W, false>), dim3(splits, Hkv, B), dim3(256), 0, stream,
                        (const bf16_t*)qkv, (Hq + 2 * Hkv) * D, (bf16_t*)out, (const bf16_t*)k_cache,
                        (const bf16_t*)v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, Hq, Hkv, page,
-                       scale_log2, window, splits, ws_acc, ws_ml, prep);
+                       scale_log2, window, splits, ws_acc, ws_ml, prep, (const float*)nullptr);
   if (splits > 1)
     hipLaunchKernelGGL(attn_decode_reduce_kernel<D>, dim3(Hkv, B), dim3(256), 0, stream, (bf16_t*)out,
-                       (const int*)nullptr, Hq, Hkv, splits, ws_acc, ws_ml);
+                       (const int*)nullptr, Hq, Hkv, splits, ws_acc, ws_ml, (const float*)nullptr);
   return q3_launch_status();
 }
 
@@ -1588,13 +1596,15 @@ extern "C" int q3_paged_attention_prompt_splits(int T, int Hq, int Hkv, int max_
 }
 
 // `splits`, `workspace`: for the sequences of few rows (q3_paged_attention_workspace);
-// `prompt_splits` (1, 2 or 4), `prompt_workspace`: for those of many.
+// `prompt_splits` (1, 2 or 4), `prompt_workspace`: for those of many. `sink` (Hq floats, or null):
+// head h's softmax has exp(sink[h]) as one more term of its denominator, unscaled and without a value.
 extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const void* k_cache,
                                   const void* v_cache, int num_pages, const int* block_table,
                                   int bt_stride, const int* cu_q, const int* kv_lens, int B, int T_, int Hq,
                                   int Hkv, int D, int page, float scale, int window, int max_q_len,
                                   int min_q_len, int max_kv_len, int dtype, int splits, float* workspace,
-                                  int prompt_splits, float* prompt_workspace, hipStream_t stream) {
+                                  int prompt_splits, float* prompt_workspace, const float* sink,
+                                  hipStream_t stream) {
   if (B <= 0 || T_ <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page <= 0 || max_q_len <= 0 || min_q_len <= 0 ||
       min_q_len > max_q_len)
     return Q3_ERR_BAD_ARGUMENT;
@@ -1610,17 +1620,17 @@ extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const 
     if (D == 64)
       return launch_fast<64>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens,
                              B, T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml,
-                             prompt_splits, prompt_workspace, stream);
+                             prompt_splits, prompt_workspace, sink, stream);
     return launch_fast<128>(q, q_stride, out, k_cache, v_cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B,
                             T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml,
-                            prompt_splits, prompt_workspace, stream);
+                            prompt_splits, prompt_workspace, sink, stream);
   }
 #ifdef Q3_SCORE_CAP
   return Q3_ERR_UNSUPPORTED;      // the capped build has the matrix-core kernels only
 #endif
   Q3_DISPATCH_DTYPE(dtype, TT, return launch_general<TT>(q, q_stride, out, k_cache, v_cache, num_pages,
                                                         block_table, bt_stride, cu_q, kv_lens, B, Hq, Hkv,
-                                                        D, page, scale, window, max_q_len, stream));
+                                                        D, page, scale, window, max_q_len, sink, stream));
   return Q3_ERR_BAD_ARGUMENT;
 }
 

@@ -1,18 +1,18 @@
 // Embedding row gather and the SwiGLU activation.
 #include "common.h"
 
-// out[t, :] = float(table[ids[t], :]). An id outside the table gives a row of
+// out[t, :] = float(table[ids[t], :]) * scale. An id outside the table gives a row of
 // zeros (the host refuses such ids before launching; this only keeps the
 // kernel inside its operands).
 template <typename T>
 __global__ void embed_rows_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                  float* __restrict__ out, int H, int V) {
+                                  float* __restrict__ out, int H, int V, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   const bool ok = id >= 0 && id < V;
   const T* row = table + (size_t)(ok ? id : 0) * H;
   float* dst = out + (size_t)t * H;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ok ? to_float(row[j]) : 0.f;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ok ? to_float(row[j]) * scale : 0.f;
 }
 
 // out[t, j] = silu(gate[t, j]) * up[t, j] for rows that interleave the two:
@@ -50,13 +50,48 @@ __global__ void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* _
   *reinterpret_cast<uint4*>(out + (size_t)t * I + j) = o.u;
 }
 
-extern "C" int q3_embed_rows(const int* ids, const void* table, float* out, int T, int H, int V,
+// A gated unit with clamped branches over rows that interleave the two (in[t, 2j] the gate's, in[t, 2j + 1]
+// the other branch's): a = in * w + bias with w = scale[scale_index[t]] (or scale[t]; 1 without a scale) and
+// a float32 bias over the interleaved columns (or none); g = min(a_gate, limit), u = clamp(a_up, -limit, limit);
+// out[t, j] = g * sigmoid(slope * g) * (u + 1). float32 throughout, rounded once; the input may be
+// float32 where the output is not (a product that left its sums unrounded).
+template <typename T, typename TO>
+__global__ void glu_clamped_kernel(const T* __restrict__ in, const float* __restrict__ bias,
+                                   const float* __restrict__ scale, const int* __restrict__ scale_index,
+                                   TO* __restrict__ out, int T_rows, int I, float limit, float slope) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= I) return;
+  const float bg = bias ? bias[2 * j] : 0.f, bu = bias ? bias[2 * j + 1] : 0.f;
+  for (int t = blockIdx.y; t < T_rows; t += gridDim.y) {
+    const float w = scale ? scale[scale_index ? scale_index[t] : t] : 1.f;
+    const T* row = in + (size_t)t * 2 * I;
+    float g = to_float(row[2 * j]) * w + bg;
+    float u = to_float(row[2 * j + 1]) * w + bu;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    out[(size_t)t * I + j] = from_float<TO>(g / (1.f + expf(-slope * g)) * (u + 1.f));
+  }
+}
+
+extern "C" int q3_glu_clamped(const void* in, const float* bias, const float* scale, const int* scale_index, void* out,
+                              int T, int I, float limit, float slope, int dtype, int out_dtype, hipStream_t stream) {
+  if (T <= 0 || I <= 0 || !(limit > 0.f) || (scale_index && !scale)) return Q3_ERR_BAD_ARGUMENT;
+  const int threads = I >= 256 ? 256 : 64;
+  const dim3 grid((I + threads - 1) / threads, T < 65535 ? T : 65535);
+  Q3_DISPATCH_DTYPE(dtype, TT, Q3_DISPATCH_DTYPE(out_dtype, TO, {
+                      hipLaunchKernelGGL((glu_clamped_kernel<TT, TO>), grid, dim3(threads), 0, stream, (const TT*)in, bias,
+                                         scale, scale_index, (TO*)out, T, I, limit, slope);
+                    }));
+  return q3_launch_status();
+}
+
+extern "C" int q3_embed_rows(const int* ids, const void* table, float* out, int T, int H, int V, float scale,
                              int table_dtype, hipStream_t stream) {
   if (T <= 0 || H <= 0 || V <= 0) return Q3_ERR_BAD_ARGUMENT;
   const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
   Q3_DISPATCH_DTYPE(table_dtype, TT,
                     hipLaunchKernelGGL(embed_rows_kernel<TT>, dim3(T), dim3(threads), 0, stream, ids,
-                                       (const TT*)table, out, H, V));
+                                       (const TT*)table, out, H, V, scale));
   return q3_launch_status();
 }
 

@@ -12,14 +12,16 @@ __device__ inline float moe_gelu(float z, int kind) {
 }
 
 // ---------------------------------------------------------------------------
-// The router's choice. One wavefront per token, from its float32 logits z (E numbers):
+// The router's choice. One wavefront per token, from its float32 logits z (E numbers). `mode` 0:
 // s = softmax(z) over all E experts, then `top` times the largest remaining score (the lowest
-// index among equals); weight_k = s_k / (sum of the chosen s + 1e-20). Every lane holds every
+// index among equals); weight_k = s_k / (sum of the chosen s + 1e-20). `mode` 1: s = sigmoid(z), each
+// expert for itself; the `top` largest are those with the largest z (chosen by z, which still tells
+// experts apart where the sigmoid has run into 1); weight_k = s_k as it is. Every lane holds every
 // reduced number and writes the same value to the same place of shared memory, so nothing here
 // waits for another lane's write.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__ logits, int n_tokens, int E, int top,
-                                                       int* __restrict__ chosen, float* __restrict__ weights) {
+                                                       int mode, int* __restrict__ chosen, float* __restrict__ weights) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x / Q3_WAVE, lane = threadIdx.x % Q3_WAVE;
   const int t = blockIdx.x * (blockDim.x / Q3_WAVE) + wave;
@@ -27,20 +29,26 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
   float* z = smem + (size_t)wave * (E + top);     // the wavefront's scores, then the chosen ones
   float* picked = z + E;
   const float* src = logits + (size_t)t * E;
-  float biggest = -INFINITY;
-  for (int e = lane; e < E; e += Q3_WAVE) biggest = fmaxf(biggest, src[e]);
-  biggest = wave_max(biggest);
-  float total = 0.f;
-  for (int e = lane; e < E; e += Q3_WAVE) {
-    const float p = expf(src[e] - biggest);
-    z[e] = p;
-    total += p;
+  float total = 1.f;
+  if (mode == 0) {
+    float biggest = -INFINITY;
+    for (int e = lane; e < E; e += Q3_WAVE) biggest = fmaxf(biggest, src[e]);
+    biggest = wave_max(biggest);
+    total = 0.f;
+    for (int e = lane; e < E; e += Q3_WAVE) {
+      const float p = expf(src[e] - biggest);
+      z[e] = p;
+      total += p;
+    }
+    total = wave_sum(total);
+  } else {
+    for (int e = lane; e < E; e += Q3_WAVE) z[e] = src[e];
   }
-  total = wave_sum(total);
   __builtin_amdgcn_wave_barrier();
+  const float nothing = mode == 0 ? -1.f : -INFINITY;     // below every score that can still be chosen
   float picked_sum = 0.f;
   for (int k = 0; k < top; ++k) {
-    float best = -1.f;
+    float best = nothing;
     int at = 0x7fffffff;
     for (int e = lane; e < E; e += Q3_WAVE) {
       const float p = z[e];
@@ -58,15 +66,16 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
         at = oa;
       }
     }
-    const float score = best / total;
+    if (at >= E) at = 0;          // logits that are no numbers: stay inside the operands
+    const float score = mode == 0 ? best / total : 1.f / (1.f + expf(-best));
     picked_sum += score;
     __builtin_amdgcn_wave_barrier();
     picked[k] = score;
-    z[at] = -2.f;               // taken
+    z[at] = mode == 0 ? -2.f : -INFINITY;               // taken
     if (lane == 0) chosen[(size_t)t * top + k] = at;
     __builtin_amdgcn_wave_barrier();
   }
-  const float inv = 1.f / (picked_sum + 1e-20f);
+  const float inv = mode == 0 ? 1.f / (picked_sum + 1e-20f) : 1.f;
   for (int k = lane; k < top; k += Q3_WAVE) weights[(size_t)t * top + k] = picked[k] * inv;
 }
 
@@ -543,7 +552,8 @@ __global__ __launch_bounds__(64 * GT_WM * 2) void moe_linear_tiles_kernel(
 }
 
 // out[t, :] = sum_k weights[t, k] * y[slot_of_pair[t * top + k], :] (+ shared[t, :]), float32 sums in
-// the order k = 0, 1, ..., the shared expert last; rounded once.
+// the order k = 0, 1, ..., the shared expert last; rounded once. Without `weights` every weight is 1
+// (experts whose inputs carried the weight).
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ slot_of_pair,
                                    const float* __restrict__ weights, const T* __restrict__ shared,
@@ -554,7 +564,7 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
   const int kept = min(top, 64);           // a token's first choices wait in shared memory, so that the rows' loads do not wait for them one by one
   if ((int)threadIdx.x < kept) {
     slots[threadIdx.x] = slot_of_pair[(size_t)t * top + threadIdx.x];
-    share[threadIdx.x] = weights[(size_t)t * top + threadIdx.x];
+    share[threadIdx.x] = weights ? weights[(size_t)t * top + threadIdx.x] : 1.f;
   }
   __syncthreads();
   const int j = blockIdx.y * blockDim.x + threadIdx.x;
@@ -562,18 +572,18 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
   float acc = 0.f;
   for (int k = 0; k < kept; ++k) acc += share[k] * to_float(y[(size_t)slots[k] * width + j]);
   for (int k = kept; k < top; ++k)
-    acc += weights[(size_t)t * top + k] * to_float(y[(size_t)slot_of_pair[(size_t)t * top + k] * width + j]);
+    acc += (weights ? weights[(size_t)t * top + k] : 1.f) * to_float(y[(size_t)slot_of_pair[(size_t)t * top + k] * width + j]);
   if (shared) acc += to_float(shared[(size_t)t * width + j]);
   out[(size_t)t * width + j] = from_float<T>(acc);
 }
 
-extern "C" int q3_moe_pick(const float* logits, int n_tokens, int E, int top, int* chosen, float* weights,
+extern "C" int q3_moe_pick(const float* logits, int n_tokens, int E, int top, int mode, int* chosen, float* weights,
                            hipStream_t stream) {
-  if (n_tokens <= 0 || E <= 0 || top <= 0 || top > E || E > 4096) return Q3_ERR_BAD_ARGUMENT;
+  if (n_tokens <= 0 || E <= 0 || top <= 0 || top > E || E > 4096 || mode < 0 || mode > 1) return Q3_ERR_BAD_ARGUMENT;
   const int waves = 4;
   const size_t smem = (size_t)waves * (E + top) * sizeof(float);
   hipLaunchKernelGGL(moe_pick_kernel, dim3((n_tokens + waves - 1) / waves), dim3(waves * Q3_WAVE), smem, stream, logits,
-                     n_tokens, E, top, chosen, weights);
+                     n_tokens, E, top, mode, chosen, weights);
   return q3_launch_status();
 }
 

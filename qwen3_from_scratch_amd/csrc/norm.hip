@@ -140,15 +140,17 @@ extern "C" int q3_rmsnorm(float* x, const void* delta, const void* weight, const
 
 // The norm behind a block that also normalises what its parts return, and behind a vector that a
 // model adds to the stream between two layers. One block per output row r (source row s):
-//   a = delta[s]                      the part's result, if there is one
+//   a = delta[s] + delta_bias         the part's result, if there is one (the bias: a product's own)
 //   a = a * rsqrt(mean(a^2) + delta_eps) * delta_weight      if delta_weight is given
 //   v = x[s] + a + bias;  if write_back: x[s] = v
-//   out[r] = v * rsqrt(mean(v^2) + eps) * weight             if out is given
+//   out[r] = v * rsqrt(mean(v^2) + eps) * weight             if out is given; without a weight
+//   out[r] = v: the stream as it is, for a sublayer that reads it without a norm in between
 // All float32; the addend is never rounded on its way into the stream. The row lives in shared
 // memory between the passes (`H` floats).
 template <typename T, typename W>
 __global__ void rmsnorm_addend_kernel(float* __restrict__ x, const T* __restrict__ delta,
                                       const W* __restrict__ delta_weight, float delta_eps,
+                                      const float* __restrict__ delta_bias,
                                       const float* __restrict__ bias, const W* __restrict__ weight,
                                       const int* __restrict__ rows, T* __restrict__ out, int H, int n_src,
                                       float eps, int write_back) {
@@ -164,7 +166,7 @@ __global__ void rmsnorm_addend_kernel(float* __restrict__ x, const T* __restrict
   if (ds && delta_weight) {
     float acc = 0.f;
     for (int j = threadIdx.x; j < H; j += blockDim.x) {
-      const float a = to_float(ds[j]);
+      const float a = to_float(ds[j]) + (delta_bias ? delta_bias[j] : 0.f);
       row[j] = a;
       acc += a * a;
     }
@@ -173,7 +175,9 @@ __global__ void rmsnorm_addend_kernel(float* __restrict__ x, const T* __restrict
   float acc = 0.f;
   for (int j = threadIdx.x; j < H; j += blockDim.x) {
     float v = xs[j];
-    if (ds) v += delta_weight ? row[j] * dscale * to_float(delta_weight[j]) : to_float(ds[j]);
+    if (ds)
+      v += delta_weight ? row[j] * dscale * to_float(delta_weight[j])
+                        : to_float(ds[j]) + (delta_bias ? delta_bias[j] : 0.f);
     if (bias) v += bias[j];
     row[j] = v;
     acc += v * v;
@@ -183,17 +187,17 @@ __global__ void rmsnorm_addend_kernel(float* __restrict__ x, const T* __restrict
   for (int j = threadIdx.x; j < H; j += blockDim.x) {
     const float v = row[j];
     if (write_back) xs[j] = v;
-    if (out) out[(size_t)r * H + j] = from_float<T>(v * scale * to_float(weight[j]));
+    if (out) out[(size_t)r * H + j] = from_float<T>(weight ? v * scale * to_float(weight[j]) : v);
   }
 }
 
 extern "C" int q3_rmsnorm_addend(float* x, const void* delta, const void* delta_weight, float delta_eps,
-                                 const float* bias, const void* weight, const int* rows, void* out, int n_out,
+                                 const float* delta_bias, const float* bias, const void* weight, const int* rows, void* out, int n_out,
                                  int n_src, int H, float eps, int act_dtype, int w_dtype, int write_back,
                                  hipStream_t stream) {
   if (n_out <= 0 || n_src <= 0 || H <= 0 || H > 36000) return Q3_ERR_BAD_ARGUMENT;
   if (write_back && rows) return Q3_ERR_BAD_ARGUMENT;
-  if (out && !weight) return Q3_ERR_BAD_ARGUMENT;
+  if (delta_bias && !delta) return Q3_ERR_BAD_ARGUMENT;
   int threads = 64;
   while (threads < 1024 && threads * 4 < H) threads *= 2;
   const size_t smem = (size_t)(32 + H) * sizeof(float);
@@ -204,7 +208,7 @@ extern "C" int q3_rmsnorm_addend(float* x, const void* delta, const void* delta_
       if (e != hipSuccess) return (int)e;
     }
     hipLaunchKernelGGL((rmsnorm_addend_kernel<TT, WW>), dim3(n_out), dim3(threads), smem, stream, x,
-                       (const TT*)delta, (const WW*)delta_weight, delta_eps, bias, (const WW*)weight, rows,
+                       (const TT*)delta, (const WW*)delta_weight, delta_eps, delta_bias, bias, (const WW*)weight, rows,
                        (TT*)out, H, n_src, eps, write_back);
     return q3_launch_status();
   }));

@@ -73,7 +73,8 @@ __global__ void softcap_prepare_kernel(const float* __restrict__ rows, long row_
 // absolute positions in steps of 64, one key a lane: score = (q . k) scale, capped as
 // cap * tanh(score / cap) when cap > 0; running maximum and sum in float32; then every lane sums
 // its columns of the values with the tile's weights. The result is divided by the sum and
-// multiplied by sigmoid(gate[t, h]) when a gate is given.
+// multiplied by sigmoid(gate[t, h]) when a gate is given. With `sink` (H floats) the sum also holds
+// exp(sink[h]), a term that has no key and no value and is not scaled.
 #define Q3_CAP_DIM_MOST 512
 #define Q3_CAP_VSLICES 8
 template <typename TA>
@@ -81,7 +82,8 @@ __global__ void __launch_bounds__(64) softcap_attention_kernel(
     const TA* __restrict__ q, const TA* __restrict__ k_cache, const TA* __restrict__ v_cache,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ seq_index,
     const int* __restrict__ positions, float scale, float cap, int window, const float* __restrict__ gate,
-    long gate_stride, TA* __restrict__ out, int H, int G, int dim, int vdim, int page, int v_transposed) {
+    long gate_stride, TA* __restrict__ out, int H, int G, int dim, int vdim, int page, int v_transposed,
+    const float* __restrict__ sink) {
   __shared__ float sq[Q3_CAP_DIM_MOST];
   __shared__ float sp[64];
   const int lane = threadIdx.x;
@@ -135,12 +137,70 @@ __global__ void __launch_bounds__(64) softcap_attention_kernel(
     __syncthreads();
   }
   const float open = gate ? 1.f / (1.f + expf(-gate[(size_t)t * gate_stride + h])) : 1.f;
+  if (sink) l += expf(sink[h] - m);
   const float norm = open / l;
 #pragma unroll
   for (int i = 0; i < Q3_CAP_VSLICES; ++i) {
     const int c = lane + 64 * i;
     if (c < vdim) out[((size_t)t * H + h) * vdim + c] = from_float<TA>(acc[i] * norm);
   }
+}
+
+// Queries, keys and values with a norm per head: one block per token, a wavefront per head in turn.
+// The row is [q: H dim | k: G dim | v: G vdim | ...] float32, or [q: H dim | ...] for a layer that
+// makes no keys of its own (`G` 0). Every head of q (of k) is divided by its own root mean square
+// and multiplied by `q_weight` (`k_weight`), dim numbers that all heads share; no rotation. q goes
+// to `q_out`, k and v into the token's place in the cache.
+template <typename TA>
+__global__ void __launch_bounds__(256) headnorm_prepare_kernel(
+    const float* __restrict__ rows, long row_stride, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, float eps, const int* __restrict__ positions, const int* __restrict__ seq_index,
+    const int* __restrict__ block_table, int table_width, TA* __restrict__ k_cache, TA* __restrict__ v_cache, int page,
+    TA* __restrict__ q_out, int H, int G, int dim, int vdim, int v_transposed) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x / Q3_WAVE, lane = threadIdx.x % Q3_WAVE, waves = blockDim.x / Q3_WAVE;
+  const float* row = rows + (size_t)t * row_stride;
+  const int nq = H * dim, nk = G * dim;
+  for (int h = wave; h < H; h += waves) {
+    const float* src = row + (size_t)h * dim;
+    float acc = 0.f;
+    for (int e = lane; e < dim; e += Q3_WAVE) acc += src[e] * src[e];
+    const float r = rsqrtf(wave_sum(acc) / (float)dim + eps);
+    for (int e = lane; e < dim; e += Q3_WAVE) q_out[(size_t)t * nq + h * dim + e] = from_float<TA>(src[e] * r * q_weight[e]);
+  }
+  if (G == 0) return;
+  const int pos = positions[t];
+  const int pg = block_table[(size_t)seq_index[t] * table_width + pos / page];
+  if (pg < 0) return;
+  const int off = pos % page;
+  for (int g = wave; g < G; g += waves) {
+    const float* src = row + nq + (size_t)g * dim;
+    float acc = 0.f;
+    for (int e = lane; e < dim; e += Q3_WAVE) acc += src[e] * src[e];
+    const float r = rsqrtf(wave_sum(acc) / (float)dim + eps);
+    for (int e = lane; e < dim; e += Q3_WAVE)
+      k_cache[(((size_t)pg * G + g) * page + off) * dim + e] = from_float<TA>(src[e] * r * k_weight[e]);
+    const float* val = row + nq + nk + (size_t)g * vdim;
+    for (int e = lane; e < vdim; e += Q3_WAVE) {
+      const size_t at = v_transposed ? (((size_t)pg * G + g) * vdim + e) * page + off
+                                     : (((size_t)pg * G + g) * page + off) * vdim + e;
+      v_cache[at] = from_float<TA>(val[e]);
+    }
+  }
+}
+
+extern "C" int q3_headnorm_prepare(const float* rows, long row_stride, const float* q_weight, const float* k_weight,
+                                   float eps, const int* positions, const int* seq_index, const int* block_table,
+                                   int table_width, void* k_cache, void* v_cache, int page, void* q_out, int T, int H,
+                                   int G, int dim, int vdim, int v_transposed, int act_dtype, hipStream_t stream) {
+  if (T <= 0 || H <= 0 || G < 0 || dim <= 0 || vdim <= 0 || !q_weight) return Q3_ERR_BAD_ARGUMENT;
+  if (G > 0 && (H % G || !k_weight || !k_cache || !v_cache || !block_table || page <= 0 || table_width <= 0))
+    return Q3_ERR_BAD_ARGUMENT;
+  Q3_DISPATCH_DTYPE(act_dtype, TA,
+                    hipLaunchKernelGGL(headnorm_prepare_kernel<TA>, dim3(T), dim3(256), 0, stream, rows, row_stride,
+                                       q_weight, k_weight, eps, positions, seq_index, block_table, table_width,
+                                       (TA*)k_cache, (TA*)v_cache, page, (TA*)q_out, H, G, dim, vdim, v_transposed));
+  return q3_launch_status();
 }
 
 // out[t, h, :] *= sigmoid(gate[t, h]) for a result that another kernel has left ungated.
@@ -180,7 +240,8 @@ extern "C" int q3_softcap_prepare(const float* rows, long row_stride, const floa
 extern "C" int q3_softcap_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
                                     int table_width, const int* seq_index, const int* positions, float scale, float cap,
                                     int window, const float* gate, long gate_stride, void* out, int T, int H, int G,
-                                    int dim, int vdim, int page, int v_transposed, int act_dtype, hipStream_t stream) {
+                                    int dim, int vdim, int page, int v_transposed, const float* sink, int act_dtype,
+                                    hipStream_t stream) {
   if (T <= 0 || H <= 0 || G <= 0 || H % G || dim <= 0 || vdim <= 0 || page <= 0 || table_width <= 0 || window < 0 ||
       H > 65535)
     return Q3_ERR_BAD_ARGUMENT;
@@ -189,6 +250,6 @@ extern "C" int q3_softcap_attention(const void* q, const void* k_cache, const vo
                     hipLaunchKernelGGL(softcap_attention_kernel<TA>, dim3(T, H), dim3(64), 0, stream, (const TA*)q,
                                        (const TA*)k_cache, (const TA*)v_cache, block_table, table_width, seq_index,
                                        positions, scale, cap, window, gate, gate_stride, (TA*)out, H, G, dim, vdim,
-                                       page, v_transposed));
+                                       page, v_transposed, sink));
   return q3_launch_status();
 }

@@ -31,6 +31,7 @@ __all__ = [
     "decode_attention",
     "decode_attention_takes",
     "swiglu",
+    "glu_clamped",
     "gelu",
     "latent_prepare",
     "headwise_linear",
@@ -38,6 +39,7 @@ __all__ = [
     "latent_attention",
     "moe_route",
     "moe_experts",
+    "moe_gated_experts",
     "embed_streams",
     "hyper_norm",
     "causal_conv",
@@ -47,6 +49,8 @@ __all__ = [
     "rglru_scan",
     "retention_scan",
     "softcap_prepare",
+    "headnorm_prepare",
+    "channel_delta",
     "softcap_attention",
     "scaled_sum",
     "linear",
@@ -247,8 +251,8 @@ def gemm_tiles(x, weight, config=0, out_dtype=None, swiglu=False, out=None, spli
     return out
 
 
-def embed_rows(ids, table, out=None):
-    """out[t, :] = float32(table[ids[t], :]). ids int32 (T,), table (V, H)."""
+def embed_rows(ids, table, out=None, scale=1.0):
+    """out[t, :] = float32(table[ids[t], :]) * scale. ids int32 (T,), table (V, H)."""
     _dev(ids, table, out)
     _need(ids.dtype == torch.int32 and ids.dim() == 1, "ids must be int32 (T,)")
     _need(table.dim() == 2 and table.dtype in _DT, "table must be (V, H) bfloat16 or float32")
@@ -258,7 +262,7 @@ def embed_rows(ids, table, out=None):
     _need(out.shape == (T, H) and out.dtype == torch.float32, "out must be float32 (T, H)")
     if T:
         _check(library("elementwise").q3_embed_rows(
-            _ptr(ids), _ptr(table), _ptr(out), T, H, V, _DT[table.dtype], _stream()), "embed_rows")
+            _ptr(ids), _ptr(table), _ptr(out), T, H, V, ctypes.c_float(scale), _DT[table.dtype], _stream()), "embed_rows")
     return out
 
 
@@ -274,6 +278,38 @@ def swiglu(gate_up, out=None):
     if T:
         _check(library("elementwise").q3_swiglu(
             _ptr(gate_up), _ptr(out), T, I, _DT[gate_up.dtype], _stream()), "swiglu")
+    return out
+
+
+def glu_clamped(gate_up, limit, slope, bias=None, scale=None, scale_index=None, out_dtype=None):
+    """A gated unit with clamped branches over rows that interleave the two (column 2j the gate's,
+    2j + 1 the other branch's): a = gate_up * w + bias; g = min(a_gate, limit), u = clamp(a_up, -limit,
+    limit); out[t, j] = g * sigmoid(slope * g) * (u + 1), float32 throughout, rounded once. `bias` float32
+    (2I,) over the interleaved columns; `scale` float32 (n,) with w = scale[scale_index[t]] (`scale_index`
+    int32 (T,)) or scale[t]: a number per row that multiplied the product's input. gate_up (T, 2I);
+    the result has `out_dtype` (gate_up's by default)."""
+    _dev(gate_up, bias, scale, scale_index)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0 and gate_up.dtype in _DT and gate_up.is_contiguous(),
+          "gate_up must be (T, 2I), contiguous, bfloat16 or float32")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    if bias is not None:
+        _f32(bias, (2 * I,), "bias")
+    if scale is not None:
+        _need(scale.dtype == torch.float32 and scale.dim() == 1 and scale.is_contiguous(), "scale must be float32 (n,)")
+        if scale_index is not None:
+            _need(scale_index.dtype == torch.int32 and scale_index.shape == (T,), "scale_index must be int32 (T,)")
+        else:
+            _need(scale.shape == (T,), "a scale without an index has one number per row")
+    else:
+        _need(scale_index is None, "an index needs a scale")
+    _need(limit > 0, "limit must be positive")
+    out_dtype = out_dtype or gate_up.dtype
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    out = torch.empty((T, I), dtype=out_dtype, device=gate_up.device)
+    if T and I:
+        _check(library("elementwise").q3_glu_clamped(
+            _ptr(gate_up), _ptr(bias), _ptr(scale), _ptr(scale_index), _ptr(out), T, I, ctypes.c_float(limit),
+            ctypes.c_float(slope), _DT[gate_up.dtype], _DT[out_dtype], _stream()), "glu_clamped")
     return out
 
 
@@ -309,16 +345,17 @@ def rmsnorm(x, weight, eps, out_dtype, delta=None, rows=None, write_back=True, o
 
 
 def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, delta_eps=0.0, bias=None, rows=None,
-                   write_back=True, out=None):
+                   write_back=True, out=None, delta_bias=None, plain=False):
     """The norm of the float32 stream behind an addend that is itself normalised first, and behind
     a vector added to every row, all in float32 and in one kernel:
 
-    a = delta[s] * rsqrt(mean(delta[s]^2) + delta_eps) * delta_weight (or delta[s] as it is without
-    `delta_weight`, or nothing); v = x[s] + a + bias; x[s] = v if `write_back`;
+    a = (delta[s] + delta_bias) * rsqrt(mean(.^2) + delta_eps) * delta_weight (or delta[s] + delta_bias
+    as it is without `delta_weight`, or nothing); v = x[s] + a + bias; x[s] = v if `write_back`;
     out[r] = v * rsqrt(mean(v^2) + eps) * weight, rounded once to `out_dtype`. With `weight` None
-    only the stream is brought up to date and None is returned. `delta` (T, H) has the activation
-    dtype, `bias` (H,) is float32, `rows` as in `rmsnorm`."""
-    _dev(x, weight, delta, delta_weight, bias, rows, out)
+    only the stream is brought up to date and None is returned, unless `plain` asks for the stream
+    itself: out[r] = v, rounded once (what a sublayer reads that has no norm before it). `delta`
+    (T, H) has the activation dtype, `bias` and `delta_bias` (H,) are float32, `rows` as in `rmsnorm`."""
+    _dev(x, weight, delta, delta_weight, bias, rows, out, delta_bias)
     _need(x.dim() == 2 and x.dtype == torch.float32, "x must be float32 (T, H)")
     T, H = x.shape
     _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
@@ -329,14 +366,16 @@ def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, del
             w_dtype = w.dtype
     if delta is not None:
         _need(delta.shape == (T, H) and delta.dtype == out_dtype, "delta must be (T, H) of the activation dtype")
-    _need(delta is not None or delta_weight is None, "a delta weight needs a delta")
-    if bias is not None:
-        _need(bias.shape == (H,) and bias.dtype == torch.float32, "bias must be float32 (H,)")
+    _need(delta is not None or (delta_weight is None and delta_bias is None), "a delta weight or bias needs a delta")
+    for b in (bias, delta_bias):
+        if b is not None:
+            _need(b.shape == (H,) and b.dtype == torch.float32, "a bias must be float32 (H,)")
+    _need(not plain or weight is None, "the plain stream is read without a weight")
     n_out = T
     if rows is not None:
         _need(rows.dtype == torch.int32 and rows.dim() == 1, "rows must be int32 (R,)")
         n_out = rows.shape[0]
-    if weight is None:
+    if weight is None and not plain:
         _need(out is None and rows is None, "without a weight there is no output")
     elif out is None:
         out = torch.empty((n_out, H), dtype=out_dtype, device=x.device)
@@ -345,9 +384,9 @@ def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, del
     write = 1 if (write_back and rows is None and (delta is not None or bias is not None)) else 0
     if n_out:
         _check(library("norm").q3_rmsnorm_addend(
-            _ptr(x), _ptr(delta), _ptr(delta_weight), ctypes.c_float(delta_eps), _ptr(bias), _ptr(weight), _ptr(rows),
-            _ptr(out), n_out, T, H, ctypes.c_float(eps), _DT[out_dtype], _DT[w_dtype or torch.float32], write, _stream()),
-            "rmsnorm_addend")
+            _ptr(x), _ptr(delta), _ptr(delta_weight), ctypes.c_float(delta_eps), _ptr(delta_bias), _ptr(bias), _ptr(weight),
+            _ptr(rows), _ptr(out), n_out, T, H, ctypes.c_float(eps), _DT[out_dtype], _DT[w_dtype or torch.float32], write,
+            _stream()), "rmsnorm_addend")
     return out
 
 
@@ -497,13 +536,19 @@ def _latent_splits(T, B, H, max_q_len, max_kv_len, window):
     return max(1, min(512 // tiles, keys // 128, 32))
 
 
-def moe_route(h, router, top, tiled=None):
-    """Per token the `top` experts with the largest softmax scores and their weights: h (T, width),
+MOE_SCORING = {"softmax": 0, "sigmoid": 1}
+
+
+def moe_route(h, router, top, tiled=None, scoring="softmax"):
+    """Per token the `top` experts with the largest scores and their weights: h (T, width),
     router (E, width) of h's dtype (`tiled`: its tile-ordered copy, if the caller keeps one). The
     logits are a product with float32 sums and a float32 result; scores, the choice and the weights
     are float32. Returns chosen int32 (T, top), in the order of falling score (the lowest index
-    among equals), and weights float32 (T, top) = score / (sum of the chosen scores + 1e-20)."""
+    among equals), and weights float32 (T, top) = score / (sum of the chosen scores + 1e-20) for
+    `scoring` "softmax" (scores = softmax over all experts); with "sigmoid" every expert's score is
+    sigmoid(z) for itself and the weights are the chosen scores as they are."""
     _dev(h, router)
+    _need(scoring in MOE_SCORING, "scoring is softmax or sigmoid")
     _need(h.dim() == 2 and router.dim() == 2 and h.shape[1] == router.shape[1] and h.dtype in _DT
           and router.dtype == h.dtype, "h (T, width) and router (E, width) of one dtype")
     T, E = h.shape[0], router.shape[0]
@@ -512,7 +557,8 @@ def moe_route(h, router, top, tiled=None):
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
     if T:
         logits = linear(h, router, out_dtype=torch.float32, tiled=tiled)
-        _check(library("moe").q3_moe_pick(_ptr(logits), T, E, top, _ptr(chosen), _ptr(weights), _stream()), "moe_route")
+        _check(library("moe").q3_moe_pick(_ptr(logits), T, E, top, MOE_SCORING[scoring], _ptr(chosen), _ptr(weights),
+                                          _stream()), "moe_route")
     return chosen, weights
 
 
@@ -567,6 +613,65 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
                                  _DT[h.dtype], stream), "moe_linear")
     _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), _ptr(weights), _ptr(shared), _ptr(out), T, width, top,
                               _DT[h.dtype], stream), "moe_combine")
+    return out
+
+
+def _moe_book(lib, chosen, E, tile_rows):
+    """The (token, choice) pairs in the order of their experts: the launch arguments that name the tiles,
+    and which pair sits in which slot and the other way round."""
+    P = chosen.numel()
+    max_tiles = -(-P // tile_rows) + E
+    book = torch.empty((E + 1 + 2 * P + 2 * max_tiles + 1,), dtype=torch.int32, device=chosen.device)
+    offsets, pair_of_slot, slot_of_pair = book[:E + 1], book[E + 1:E + 1 + P], book[E + 1 + P:E + 1 + 2 * P]
+    at = E + 1 + 2 * P
+    tile_expert, tile_first, n_tiles = book[at:at + max_tiles], book[at + max_tiles:at + 2 * max_tiles], book[at + 2 * max_tiles:]
+    _check(lib.q3_moe_align(_ptr(chosen), P, E, tile_rows, _ptr(offsets), _ptr(pair_of_slot), _ptr(slot_of_pair),
+                            _ptr(tile_expert), _ptr(tile_first), _ptr(n_tiles), _stream()), "moe_align")
+    return (_ptr(tile_expert), _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles), pair_of_slot, slot_of_pair
+
+
+def moe_gated_experts(h, chosen, weights, gate_up, down, limit, slope):
+    """sum_k down[e] y, y = glu(gate_up[e] (weights[t, k] h[t])), e = chosen[t, k]: experts that are gated
+    units with clamped branches (`glu_clamped`), whose weight multiplies the expert's input, not its
+    result. h (T, width), gate_up (E, 2 ff, width) with rows 2j the gate's and 2j + 1 the other branch's,
+    down (E, width, ff); returns (T, width). The weight enters behind the first product, which is
+    linear in its input, in float32 and before the clamps; a token's sum is formed in float32 in the
+    order of its choices."""
+    _dev(h, chosen, weights, gate_up, down)
+    T, width = h.shape
+    E, ff = down.shape[0], down.shape[2]
+    top = chosen.shape[1]
+    _need(h.dtype in _DT and gate_up.dtype == h.dtype and down.dtype == h.dtype and gate_up.shape == (E, 2 * ff, width)
+          and down.shape == (E, width, ff), "gate_up (E, 2 ff, width) and down (E, width, ff) of h's dtype")
+    _need(chosen.shape == (T, top) and chosen.dtype == torch.int32 and weights.shape == (T, top)
+          and weights.dtype == torch.float32 and weights.is_contiguous(), "chosen int32 (T, top), weights float32 (T, top)")
+    out = torch.empty((T, width), dtype=h.dtype, device=h.device)
+    if not T:
+        return out
+    lib = library("moe")
+    P = T * top
+    cores = h.dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
+    many = 3 if width % 64 == 0 and ff % 64 == 0 else 2
+    tile_rows = lib.q3_moe_tile_rows((many if P >= 96 * E else 1) if cores else 0)
+    tiles, pair_of_slot, slot_of_pair = _moe_book(lib, chosen, E, tile_rows)
+    both = torch.empty((P, 2 * ff), dtype=h.dtype, device=h.device)
+    y = torch.empty((P, width), dtype=h.dtype, device=h.device)
+    stream = _stream()
+    if cores:
+        _check(lib.q3_moe_linear_mma(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(both), *tiles, 2 * ff, width,
+                                     -1, tile_rows, stream), "moe_linear")
+    else:
+        _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(both), *tiles, 2 * ff, width, -1,
+                                 _DT[h.dtype], stream), "moe_linear")
+    hidden = glu_clamped(both, limit, slope, scale=weights.view(-1), scale_index=pair_of_slot)
+    if cores:
+        _check(lib.q3_moe_linear_mma(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff,
+                                     -1, tile_rows, stream), "moe_linear")
+    else:
+        _check(lib.q3_moe_linear(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff, -1,
+                                 _DT[h.dtype], stream), "moe_linear")
+    _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), None, None, _ptr(out), T, width, top, _DT[h.dtype], stream),
+           "moe_combine")
     return out
 
 
@@ -872,24 +977,110 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
     return q
 
 
+def headnorm_prepare(rows, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, positions, seq_index, out_dtype,
+                     block_table=None, k_cache=None, v_cache=None, values_transposed=False):
+    """Queries, keys and values of a step from the float32 rows of their joint product, with a norm per
+    head and no rotation.
+
+    rows float32 (T, n) laid out [q: heads dim | k: kv_heads dim | v: kv_heads vdim | ...]; every head
+    of q and of k is divided by its own root mean square (eps inside the root) and multiplied by
+    `q_weight` or `k_weight`, float32 (dim,), shared by the heads. Returns q (T, heads, dim) of
+    `out_dtype`; keys and values go to their positions in the cache, laid out as for
+    `softcap_prepare`. With `kv_heads` 0 the rows hold no keys and values (a layer that reads
+    another layer's) and nothing is written."""
+    _dev(q_weight, k_weight, positions, seq_index, block_table, k_cache, v_cache)
+    _need(rows.is_cuda and rows.dim() == 2 and rows.dtype == torch.float32 and rows.stride(1) == 1, "rows must be float32 (T, n)")
+    T = rows.shape[0]
+    _need(heads > 0 and kv_heads >= 0 and (kv_heads == 0 or heads % kv_heads == 0), "kv_heads divides heads (or is 0)")
+    _need(rows.shape[1] >= heads * dim + kv_heads * (dim + vdim), "rows hold q, k and v")
+    _f32(q_weight, (dim,), "q_weight")
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and seq_index.dtype == torch.int32
+          and seq_index.shape == (T,), "positions and seq_index must be int32 (T,)")
+    page = width = 0
+    if kv_heads:
+        _f32(k_weight, (dim,), "k_weight")
+        _need(k_cache is not None and v_cache is not None and block_table is not None and block_table.dtype == torch.int32
+              and block_table.dim() == 2, "keys of its own need a key cache, a value cache and an int32 block table")
+        page, width = k_cache.shape[2], block_table.shape[1]
+        _need(k_cache.dim() == 4 and k_cache.shape[1:] == (kv_heads, page, dim) and v_cache.dim() == 4
+              and v_cache.shape[1:] == ((kv_heads, vdim, page) if values_transposed else (kv_heads, page, vdim))
+              and k_cache.dtype == out_dtype and v_cache.dtype == out_dtype and k_cache.is_contiguous()
+              and v_cache.is_contiguous(),
+              "keys (pages, kv_heads, page, dim) and values (pages, kv_heads, page, vdim) of out_dtype")
+    q = torch.empty((T, heads, dim), dtype=out_dtype, device=rows.device)
+    if T:
+        _check(library("softcap").q3_headnorm_prepare(
+            _ptr(rows), ctypes.c_long(rows.stride(0)), _ptr(q_weight), _ptr(k_weight) if kv_heads else None,
+            ctypes.c_float(eps), _ptr(positions), _ptr(seq_index), _ptr(block_table) if kv_heads else None, width,
+            _ptr(k_cache) if kv_heads else None, _ptr(v_cache) if kv_heads else None, page, _ptr(q), T, heads, kv_heads,
+            dim, vdim, 1 if values_transposed else 0, _DT[out_dtype], _stream()), "headnorm_prepare")
+    return q
+
+
+def channel_delta(conv, b_logits, a_logits, gate, dt_bias, a_log, norm_weight, eps, unit_eps, state, slots, cu_seqlens_q,
+                  heads, kv_heads, dim, vdim, out_dtype):
+    """The gated delta rule with a decay per head and key channel over a packed step, float32.
+
+    conv float32 (T, 2 kv_heads dim + heads vdim) contiguous: [q | k | v] behind their convolutions and
+    activations; head h reads q and k of group h // (heads / kv_heads). b_logits (T, heads), a_logits
+    (T, heads dim) and gate (T, heads vdim): float32, rows possibly apart. q and k become unit vectors
+    per head, x / sqrt(sum(x^2) + unit_eps), q also times dim^(-1/2); beta = sigmoid(b_logits);
+    g = exp(-exp(a_log[h]) softplus(a_logits + dt_bias)), a number per head and key channel. Per head
+
+        S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q;
+
+    o is divided by the root mean square of the head's vdim numbers (eps inside the root), multiplied
+    by `norm_weight` (vdim,) and by sigmoid(gate). state float32 (slots, heads vdim dim) laid out (head,
+    column, row), continued and brought up to date. Returns (T, heads vdim) of `out_dtype`."""
+    _dev(conv, dt_bias, a_log, norm_weight)
+    T = conv.shape[0]
+    _need(heads > 0 and kv_heads > 0 and heads % kv_heads == 0 and 0 < dim <= 256 and vdim > 0,
+          "kv_heads divides heads; dim at most 256")
+    _f32(conv, (T, 2 * kv_heads * dim + heads * vdim), "conv")
+    for t, n, what in ((b_logits, heads, "b_logits"), (a_logits, heads * dim, "a_logits"), (gate, heads * vdim, "gate")):
+        _rows_view(t, what)
+        _need(t.shape == (T, n) and t.dtype == torch.float32, "%s must be float32 (T, %d)" % (what, n))
+    _f32(dt_bias, (heads * dim,), "dt_bias")
+    _f32(a_log, (heads,), "a_log")
+    _f32(norm_weight, (vdim,), "norm_weight")
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    B = _sequences(slots, cu_seqlens_q, state, heads * dim * vdim, "channel_delta")
+    out = torch.empty((T, heads * vdim), dtype=out_dtype, device=conv.device)
+    if T:
+        lib = library("delta")
+        lib.q3_channel_delta_workspace.restype = ctypes.c_long
+        work = torch.empty(lib.q3_channel_delta_workspace(T, heads, dim, vdim), dtype=torch.float32, device=conv.device)
+        _check(lib.q3_channel_delta(
+            _ptr(conv), _ptr(b_logits), ctypes.c_long(b_logits.stride(0)), _ptr(a_logits), ctypes.c_long(a_logits.stride(0)),
+            _ptr(gate), ctypes.c_long(gate.stride(0)), _ptr(dt_bias), _ptr(a_log), _ptr(norm_weight), ctypes.c_float(eps),
+            ctypes.c_float(unit_eps), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(out),
+            _ptr(work), T, B, heads, kv_heads, dim, vdim, _DT[out_dtype], _stream()), "channel_delta")
+    return out
+
+
 def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, seq_index, positions, max_q_len,
                       max_kv_len, scale, softcap, window=0, gate=None, values_transposed=False, min_q_len=1,
-                      max_kv_len_of_many=None):
+                      max_kv_len_of_many=None, sink=None):
     """Causal softmax attention over a paged cache whose keys and values differ in size.
 
     q (T, heads, dim); keys (pages, kv_heads, page, dim), values (pages, kv_heads, page, vdim); the
     token at row t of sequence seq_index[t] sits at positions[t] and sees the keys at positions
     j <= positions[t] (with `window` > 0 only the last `window` of them). score = (q . k) scale, then
     softcap * tanh(score / softcap) if softcap > 0; softmax in float32. `gate` float32 (T, heads),
-    rows possibly apart: head h's result is multiplied by sigmoid(gate[t, h]). Returns (T, heads vdim).
+    rows possibly apart: head h's result is multiplied by sigmoid(gate[t, h]). `sink` float32 (heads,):
+    head h's softmax has exp(sink[h]) as one more term of its denominator, a key that is always seen, is
+    not scaled and has no value. Returns (T, heads vdim).
 
     With `values_transposed` the values are (pages, kv_heads, vdim, page), and bfloat16 with equal key
     and value sizes of 64 or 128 then runs on the matrix cores, through the kernels of
     `paged_attention` (`min_q_len` and `max_kv_len_of_many` are theirs); everything else takes a
     general kernel of one wavefront per (token, head)."""
-    _dev(q, k_cache, v_cache, block_table, seq_index, positions)
+    _dev(q, k_cache, v_cache, block_table, seq_index, positions, sink)
     _need(q.dim() == 3 and q.dtype in _DT, "q must be (T, heads, dim)")
     T, H, dim = q.shape
+    if sink is not None:
+        _f32(sink, (H,), "sink")
     _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[3] == dim and k_cache.shape[:2] == v_cache.shape[:2]
           and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "keys (pages, G, page, dim), values (pages, G, page, vdim)")
     G, page = k_cache.shape[1], k_cache.shape[2]
@@ -907,7 +1098,8 @@ def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, s
     if T and values_transposed and dim == vdim and q.dtype == torch.bfloat16 \
             and library("attention").q3_paged_attention_fast_path(H, G, dim, page, _DT[q.dtype]):
         out = paged_attention(q, H, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, max_q_len, max_kv_len, scale,
-                              window=window, min_q_len=min_q_len, max_kv_len_of_many=max_kv_len_of_many, softcap=softcap)
+                              window=window, min_q_len=min_q_len, max_kv_len_of_many=max_kv_len_of_many, softcap=softcap,
+                              sink=sink)
         if gate is not None:
             _check(library("softcap").q3_gate_heads(_ptr(out), _ptr(gate), ctypes.c_long(stride), T, H, vdim,
                                                     _DT[q.dtype], _stream()), "gate_heads")
@@ -917,8 +1109,8 @@ def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, s
         _check(library("softcap").q3_softcap_attention(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_index),
             _ptr(positions), ctypes.c_float(scale), ctypes.c_float(softcap), int(window), _ptr(gate),
-            ctypes.c_long(stride), _ptr(out), T, H, G, dim, vdim, page, 1 if values_transposed else 0, _DT[q.dtype],
-            _stream()), "softcap_attention")
+            ctypes.c_long(stride), _ptr(out), T, H, G, dim, vdim, page, 1 if values_transposed else 0, _ptr(sink),
+            _DT[q.dtype], _stream()), "softcap_attention")
     return out
 
 
@@ -1018,10 +1210,12 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
 
 
 def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens,
-                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1, max_kv_len_of_many=None, softcap=0.0):
+                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1, max_kv_len_of_many=None, softcap=0.0,
+                    sink=None):
     """Causal softmax attention of packed query rows over paged keys and values.
     `softcap` > 0: a score s enters the softmax as softcap * tanh(s * scale / softcap); that form
     exists for the sizes the matrix cores take (a second build of the same kernels) and no other.
+    `sink` float32 (Hq,): exp(sink[h]) joins the denominator of head h's softmax (no key, no value).
 
     q is (T, Hq, D) seen through a row stride (a view of the qkv buffer is
     fine). Keys are cached as (pages, Hkv, page, D), values as
@@ -1040,7 +1234,9 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
     runs on the matrix cores; everything else (float32, other head sizes in
     steps of 16 up to 256, other page sizes) takes the general kernel.
     """
-    _dev(k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, out)
+    _dev(k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, out, sink)
+    if sink is not None:
+        _f32(sink, (num_q_heads,), "sink")
     _need(q.is_cuda and q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2],
           "q must be (T, Hq, D) with contiguous heads")
     T, Hq, D = q.shape
@@ -1087,7 +1283,7 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
             _ptr(q), q.stride(0), _ptr(out), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
             _ptr(block_table), block_table.shape[1], _ptr(cu_seqlens_q), _ptr(kv_lens),
             B, T, Hq, Hkv, D, page, ctypes.c_float(scale), int(window), int(max_q_len), int(min_q_len),
-            int(max_kv_len), _DT[q.dtype], splits, _ptr(workspace), prompt_splits, _ptr(prompt_workspace),
+            int(max_kv_len), _DT[q.dtype], splits, _ptr(workspace), prompt_splits, _ptr(prompt_workspace), _ptr(sink),
             _stream()),
             "paged_attention")
     return out

@@ -30,7 +30,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-MODULES = ("elementwise", "norm", "rotary", "attention", "attention_capped", "latent", "moe", "hyper", "recurrent", "softcap", "gemm", "matmul",
+MODULES = ("elementwise", "norm", "rotary", "attention", "attention_capped", "latent", "moe", "hyper", "recurrent", "delta", "softcap", "gemm", "matmul",
            "sampling", "probes")
 # what a module links besides the HIP runtime
 LINKS = {"matmul": ["-lhipblaslt"]}

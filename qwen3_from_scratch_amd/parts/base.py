@@ -74,6 +74,15 @@ class TensorShape(tuple):
         return self
 
 
+class AnySize(int):
+    """A size in a tensor's shape that the checkpoint decides and no configuration names (the inner
+    size of a product through a narrow middle, say): whatever the stored tensor has there is
+    right, and the part reads it off the tensor when it loads. Its value as a number is what
+    random weights are made with."""
+
+    any_size = True
+
+
 class Part:
     """Base class. `prefix` is the checkpoint name prefix of the part's tensors."""
 
@@ -151,13 +160,30 @@ class StreamAddend:
     activation dtype, a part's result, which is first normalised by its root mean square with
     `weight` and `eps` if `weight` is given (a block that also normalises what its parts return);
     and `bias` (width,) float32, one vector for every row (what a model adds to the stream
-    between two layers). Either may be None. A norm that takes it as `delta` does the whole sum
-    in float32 in its own kernel, so the addend is never rounded on its way into the stream."""
+    between two layers). Either may be None. `values_bias` (width,) float32 belongs to the part's
+    result itself (the bias of its last product, see `BiasedRows`) and joins `values` before their
+    norm. A norm that takes it as `delta` does the whole sum in float32 in its own kernel, so the
+    addend is never rounded on its way into the stream."""
 
     values: torch.Tensor = None
     weight: torch.Tensor = None
     eps: float = 0.0
     bias: torch.Tensor = None
+    values_bias: torch.Tensor = None
+
+
+@dataclass
+class BiasedRows:
+    """A part's result whose last product has a bias that is not added yet: `values` (T, width) in
+    the activation dtype and `bias` (width,) float32. A block that hands results on as a
+    `StreamAddend` lets the bias ride along, so that it is added in float32 by the kernel that
+    takes the result into the stream; `finished()` adds it on the spot for anyone else."""
+
+    values: torch.Tensor
+    bias: torch.Tensor
+
+    def finished(self):
+        return (self.values.float() + self.bias).to(self.values.dtype)
 
 
 @dataclass

@@ -3,7 +3,7 @@
 from ..config.registry import register_part
 import torch
 
-from .base import HyperAddend, Part, TensorShape, UnscaledRows
+from .base import BiasedRows, HyperAddend, Part, TensorShape, UnscaledRows
 
 
 def _says(part, what):
@@ -89,6 +89,8 @@ class SandwichBlock(Part):
     def _behind(norm, values):
         if hasattr(norm, "as_addend"):
             return norm.as_addend(values)
+        if isinstance(values, BiasedRows):
+            values = values.finished()
         return norm.forward(values.float())
 
     def forward(self, x, pending, batch, cache, next_norm=None):

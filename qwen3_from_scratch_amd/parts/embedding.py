@@ -9,15 +9,18 @@ from .base import Part, StreamAddend, UnscaledRows
 
 @register_part("embedding", "token")
 class TokenEmbedding(Part):
-    """x[t] = E[ids[t]], no scaling, no padding row
+    """x[t] = E[ids[t]] * scale, no padding row; `scale` is 1 unless the architecture says otherwise
     (src/qwen3_from_scratch/models/qwen3.py:17-19,45). With `copies` the residual starts as
     that many equal streams, (T, copies, hidden_size), for blocks that keep several."""
 
     graph_safe = True
 
-    def __init__(self, prefix, precision, device, vocab_size, hidden_size, leaf="weight", copies=0):
+    def __init__(self, prefix, precision, device, vocab_size, hidden_size, leaf="weight", copies=0, scale=1.0):
         super().__init__(prefix, precision, device)
         self.copies = int(copies)
+        self.scale = float(scale)
+        if self.copies and self.scale != 1.0:
+            raise ValueError("a residual that starts as several streams has no scale on its embedding")
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.leaf = leaf
@@ -32,7 +35,7 @@ class TokenEmbedding(Part):
     def forward(self, token_ids):
         if self.copies:
             return ops.embed_streams(token_ids, self.weight, self.copies)
-        return ops.embed_rows(token_ids, self.weight)
+        return ops.embed_rows(token_ids, self.weight, scale=self.scale)
 
 
 @register_part("embedding", "pass_vectors")
@@ -66,5 +69,6 @@ class PassVectors(Part):
         if isinstance(pending, StreamAddend):
             if pending.bias is not None:
                 raise ValueError("two vectors wait for the same place of the stream")
-            return StreamAddend(values=pending.values, weight=pending.weight, eps=pending.eps, bias=row)
+            return StreamAddend(values=pending.values, weight=pending.weight, eps=pending.eps, bias=row,
+                                values_bias=pending.values_bias)
         return StreamAddend(values=pending, bias=row)

@@ -4,7 +4,7 @@ import torch
 
 from .. import ops
 from ..config.registry import register_part
-from .base import HyperAddend, NormSink, Part, StreamAddend, TensorShape
+from .base import BiasedRows, HyperAddend, NormSink, Part, StreamAddend, TensorShape
 
 
 @register_part("norm", "rms")
@@ -36,13 +36,16 @@ class RMSNorm(Part):
         if isinstance(delta, StreamAddend):
             return ops.rmsnorm_addend(x, self.weight, self.eps, self.precision.act, delta=delta.values,
                                       delta_weight=delta.weight, delta_eps=delta.eps, bias=delta.bias, rows=rows,
-                                      write_back=rows is None)
+                                      write_back=rows is None, delta_bias=delta.values_bias)
         return ops.rmsnorm(x, self.weight, self.eps, self.precision.act, delta=delta,
                            rows=rows, write_back=rows is None)
 
     def as_addend(self, values):
-        """`values` (a part's result) as what the stream still lacks, to be normalised by this norm
-        on its way in: the norm that reads the stream next does both in one kernel."""
+        """`values` (a part's result, a tensor or `BiasedRows`) as what the stream still lacks, to be
+        normalised by this norm on its way in: the norm that reads the stream next does both in one
+        kernel."""
+        if isinstance(values, BiasedRows):
+            return StreamAddend(values=values.values, weight=self.weight, eps=self.eps, values_bias=values.bias)
         return StreamAddend(values=values, weight=self.weight, eps=self.eps)
 
     def sink_for(self, x):
@@ -56,6 +59,28 @@ class RMSNorm(Part):
         if not 1 <= rows <= ops.FUSED_ROWS_MOST or self.size % (16 if rows <= ops.FUSED_ROWS_FEW else 64):
             return None
         return NormSink(x, self.weight, self.eps, self.size)
+
+
+@register_part("norm", "none")
+class StreamReader(Part):
+    """No norm at all, in a norm's place: y = x, the float32 residual stream rounded once to the
+    activation dtype, for sublayers that read the stream as it is (a layer that normalises only
+    what its parts return). Like the norms it folds the pending addition into its pass: a
+    `StreamAddend` is normalised, added into the stream and the sum read in one kernel. It has no
+    tensors; `size` is the stream's width."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device, size):
+        super().__init__(prefix, precision, device)
+        self.size = size
+
+    def forward(self, x, delta=None, rows=None):
+        if not isinstance(delta, StreamAddend):
+            delta = StreamAddend(values=delta)
+        return ops.rmsnorm_addend(x, None, 0.0, self.precision.act, delta=delta.values, delta_weight=delta.weight,
+                                  delta_eps=delta.eps, bias=delta.bias, rows=rows, write_back=rows is None,
+                                  delta_bias=delta.values_bias, plain=True)
 
 
 @register_part("norm", "layer")

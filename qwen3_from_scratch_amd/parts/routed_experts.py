@@ -59,3 +59,53 @@ class RoutedExperts(Part):
         if self.shared_ff:
             shared = self.shared_down.forward(ops.gelu(self.shared_up.forward(x), self.activation))
         return ops.moe_experts(x, chosen, weights, self.up, self.down, shared=shared, activation=self.activation)
+
+
+@register_part("feed_forward", "gated_experts")
+class GatedExperts(Part):
+    """z = W_router h (float32), s = sigmoid(z), every expert for itself; a token's `top` experts are
+    those with the largest scores (the lowest index among equals) and their weights are those
+    scores as they are. Each expert is a gated unit with clamped branches and no biases,
+    g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), W_down (g sigmoid(slope g) (u + 1)),
+    and its weight multiplies its input, not its result: the layer's result is the sum of
+    expert_e(s_e h) over the chosen e.
+
+    Tensors: router (experts, hidden), e<i>.gate and e<i>.up (expert_ff, hidden), e<i>.down (hidden,
+    expert_ff). The experts' matrices are kept stacked, gate and up as one with their rows
+    interleaved, (experts, 2 ff, hidden), and (experts, hidden, ff); tokens are never counted on
+    the host, so a step is launches only."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device, hidden_size, experts, top, expert_ff, limit, slope=1.702):
+        super().__init__(prefix, precision, device)
+        if not 1 <= top <= experts:
+            raise ValueError("top (%d) must lie in 1..experts (%d)" % (top, experts))
+        if not limit > 0:
+            raise ValueError("limit must be positive")
+        self.hidden_size, self.experts, self.top, self.expert_ff = hidden_size, experts, top, expert_ff
+        self.limit, self.slope = float(limit), float(slope)
+        self.router = self.gate_up = self.down = None
+
+    def tensors(self):
+        W = self.hidden_size
+        names = {self._name("router"): (self.experts, W)}
+        for e in range(self.experts):
+            names[self._name("e%d.gate" % e)] = (self.expert_ff, W)
+            names[self._name("e%d.up" % e)] = (self.expert_ff, W)
+            names[self._name("e%d.down" % e)] = (W, self.expert_ff)
+        return names
+
+    def load(self, fetch):
+        act, E, ff, W = self.precision.act, self.experts, self.expert_ff, self.hidden_size
+        self.router = LinearWeight(fetch(self._name("router"), act), self.precision)
+        gate_up = torch.empty((E, 2 * ff, W), dtype=act, device=self.device)
+        for e in range(E):
+            gate_up[e, 0::2].copy_(fetch(self._name("e%d.gate" % e), act, keep=False))
+            gate_up[e, 1::2].copy_(fetch(self._name("e%d.up" % e), act, keep=False))
+        self.gate_up = gate_up
+        self.down = torch.stack([fetch(self._name("e%d.down" % e), act, keep=False) for e in range(E)]).contiguous()
+
+    def forward(self, x, batch=None):
+        chosen, weights = ops.moe_route(x, self.router.weight, self.top, tiled=self.router.tiled, scoring="sigmoid")
+        return ops.moe_gated_experts(x, chosen, weights, self.gate_up, self.down, self.limit, self.slope)

@@ -130,8 +130,9 @@ def check_tensors(source, expected, ignorable=()):
     unexpected = have - want - set(ignorable)
     wrong = []
     for name in want & have:
-        found = tuple(source.shape(name))
-        if found != tuple(expected[name]):
-            wrong.append((name, tuple(expected[name]), found))
+        found, wanted = tuple(source.shape(name)), tuple(expected[name])
+        # a size the part leaves to the checkpoint (it says `any_size`) fits whatever is found there
+        if len(found) != len(wanted) or any(f != w and not getattr(w, "any_size", False) for f, w in zip(found, wanted)):
+            wrong.append((name, wanted, found))
     if missing or unexpected or wrong:
         raise WeightError(missing, unexpected, wrong, source.where)

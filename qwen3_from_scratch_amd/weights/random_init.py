@@ -41,7 +41,7 @@ class RandomWeights(TensorSource):
         return tuple(self._expected[name])
 
     def get(self, name, device):
-        shape = self.shape(name)
+        shape = tuple(int(n) for n in self.shape(name))
         on = torch.device(self.generate_on) if self.generate_on is not None else torch.device("cpu")
         gen = torch.Generator(device=on)
         gen.manual_seed(_tensor_seed(self.seed, name))

@@ -12,8 +12,8 @@ import math
 import torch
 
 
-def embed_rows(ids, table, out=None):
-    res = table[ids.long()].float()
+def embed_rows(ids, table, out=None, scale=1.0):
+    res = table[ids.long()].float() * scale
     if out is not None:
         out.copy_(res)
         return out
@@ -177,10 +177,12 @@ def sample(logits, temperature, top_k, seed, counter, out=None, any_top_k=True):
 
 
 def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, delta_eps=0.0, bias=None, rows=None,
-                   write_back=True, out=None):
+                   write_back=True, out=None, delta_bias=None, plain=False):
     src = x if rows is None else x[rows.long()]
     if delta is not None:
         d = (delta if rows is None else delta[rows.long()]).float()
+        if delta_bias is not None:
+            d = d + delta_bias
         if delta_weight is not None:
             d = d * torch.rsqrt((d * d).mean(dim=-1, keepdim=True) + delta_eps) * delta_weight.float()
         src = src + d
@@ -188,13 +190,28 @@ def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, del
         src = src + bias
     if write_back and rows is None and (delta is not None or bias is not None):
         x.copy_(src)
-    if weight is None:
+    if weight is None and not plain:
         return None
-    res = (src * torch.rsqrt((src * src).mean(dim=-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
+    if plain:
+        res = src.to(out_dtype)
+    else:
+        res = (src * torch.rsqrt((src * src).mean(dim=-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
     if out is not None:
         out.copy_(res)
         return out
     return res
+
+
+def glu_clamped(gate_up, limit, slope, bias=None, scale=None, scale_index=None, out_dtype=None):
+    a = gate_up.float()
+    if scale is not None:
+        w = scale[scale_index.long()] if scale_index is not None else scale
+        a = a * w[:, None]
+    if bias is not None:
+        a = a + bias
+    g = torch.clamp(a[:, 0::2], max=limit)
+    u = torch.clamp(a[:, 1::2], min=-limit, max=limit)
+    return (g * torch.sigmoid(slope * g) * (u + 1.0)).to(out_dtype or gate_up.dtype)
 
 
 GELU_KINDS = {"erf": 0, "tanh": 1}
@@ -277,10 +294,25 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
     return res.to(q.dtype)
 
 
-def moe_route(h, router, top, tiled=None):
-    s = torch.softmax(h.float() @ router.float().T, dim=-1)
+def moe_route(h, router, top, tiled=None, scoring="softmax"):
+    z = h.float() @ router.float().T
+    if scoring == "sigmoid":
+        best, chosen = torch.topk(z, top, dim=-1)
+        return chosen.to(torch.int32), torch.sigmoid(best)
+    s = torch.softmax(z, dim=-1)
     best, chosen = torch.topk(s, top, dim=-1)
     return chosen.to(torch.int32), best / (best.sum(dim=-1, keepdim=True) + 1e-20)
+
+
+def moe_gated_experts(h, chosen, weights, gate_up, down, limit, slope):
+    T, top = chosen.shape
+    out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
+    for k in range(top):
+        e = chosen[:, k].long()
+        both = torch.einsum("ti,tfi->tf", h.float(), gate_up[e].float()).to(h.dtype)
+        hidden = glu_clamped(both, limit, slope, scale=weights[:, k].contiguous())
+        out += torch.einsum("tf,twf->tw", hidden.float(), down[e].float()).to(h.dtype).float()
+    return out.to(h.dtype)
 
 
 def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
@@ -456,9 +488,55 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
     return q.to(out_dtype).contiguous()
 
 
+def headnorm_prepare(rows, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, positions, seq_index, out_dtype,
+                     block_table=None, k_cache=None, v_cache=None, values_transposed=False):
+    T = rows.shape[0]
+    nq, nk = heads * dim, kv_heads * dim
+    q = rows[:, :nq].float().view(T, heads, dim)
+    q = q * torch.rsqrt((q * q).mean(dim=-1, keepdim=True) + eps) * q_weight.float()
+    if kv_heads:
+        k = rows[:, nq:nq + nk].float().view(T, kv_heads, dim)
+        k = k * torch.rsqrt((k * k).mean(dim=-1, keepdim=True) + eps) * k_weight.float()
+        v = rows[:, nq + nk:nq + nk + kv_heads * vdim].float().reshape(T, kv_heads, vdim)
+        page = k_cache.shape[2]
+        pos = positions.long()
+        pages = block_table[seq_index.long(), pos // page].long()
+        k_cache[pages, :, pos % page] = k.to(k_cache.dtype)
+        if values_transposed:
+            v_cache[pages, :, :, pos % page] = v.to(v_cache.dtype)
+        else:
+            v_cache[pages, :, pos % page] = v.to(v_cache.dtype)
+    return q.to(out_dtype).contiguous()
+
+
+def channel_delta(conv, b_logits, a_logits, gate, dt_bias, a_log, norm_weight, eps, unit_eps, state, slots, cu_seqlens_q,
+                  heads, kv_heads, dim, vdim, out_dtype):
+    T = conv.shape[0]
+    H, G, d, dv = heads, kv_heads, dim, vdim
+    q = conv[:, :G * d].view(T, G, d)
+    k = conv[:, G * d:2 * G * d].view(T, G, d)
+    v = conv[:, 2 * G * d:].view(T, H, dv)
+    q = q * torch.rsqrt((q * q).sum(dim=-1, keepdim=True) + unit_eps) * d ** -0.5
+    k = k * torch.rsqrt((k * k).sum(dim=-1, keepdim=True) + unit_eps)
+    q, k = q.repeat_interleave(H // G, dim=1), k.repeat_interleave(H // G, dim=1)
+    beta = torch.sigmoid(b_logits)
+    decay = torch.exp(-torch.exp(a_log)[None, :, None] * torch.nn.functional.softplus((a_logits + dt_bias).view(T, H, d)))
+    o = torch.empty((T, H, dv), dtype=torch.float32, device=conv.device)
+    for first, last, slot in _sequences(cu_seqlens_q, slots):
+        S = state[slot].view(H, dv, d).transpose(1, 2).clone()       # kept (head, column, row)
+        for t in range(first, last):
+            S = decay[t][:, :, None] * S
+            u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+            S = S + k[t][:, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S.transpose(1, 2).reshape(-1)
+    o = o * torch.rsqrt((o * o).mean(dim=-1, keepdim=True) + eps) * norm_weight * torch.sigmoid(gate.view(T, H, dv))
+    return o.reshape(T, H * dv).to(out_dtype)
+
+
 def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, seq_index, positions, max_q_len,
                       max_kv_len, scale, softcap, window=0, gate=None, values_transposed=False, min_q_len=1,
-                      max_kv_len_of_many=None):
+                      max_kv_len_of_many=None, sink=None):
     T, H, dim = q.shape
     if values_transposed:
         v_cache = v_cache.transpose(2, 3)
@@ -484,7 +562,11 @@ def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, s
             if softcap > 0:
                 s = softcap * torch.tanh(s / softcap)
             s = s.masked_fill(hidden, float("-inf"))
-            res[q0:q1, h] = torch.softmax(s, dim=-1) @ V[h // (H // G)]
+            if sink is not None:
+                s = torch.cat((s, sink[h].float().expand(n, 1)), dim=-1)
+                res[q0:q1, h] = torch.softmax(s, dim=-1)[:, :-1] @ V[h // (H // G)]
+            else:
+                res[q0:q1, h] = torch.softmax(s, dim=-1) @ V[h // (H // G)]
     if gate is not None:
         res = res * torch.sigmoid(gate.float())[:, :, None]
     return res.reshape(T, H * vdim).to(q.dtype)
@@ -494,7 +576,7 @@ def scaled_sum(a, alpha, b, beta):
     return (alpha * a.float() + beta * b.float()).to(a.dtype)
 
 
-ALL = ("embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
+ALL = ("glu_clamped", "moe_gated_experts", "headnorm_prepare", "channel_delta", "embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
        "paged_attention", "decode_attention_takes", "linear", "linear_swiglu", "tile_weight", "sample",
        "rmsnorm_addend", "gelu", "GELU_KINDS", "latent_prepare", "headwise_linear", "rotate_heads", "latent_attention",
        "moe_route", "moe_experts", "embed_streams", "hyper_norm", "causal_conv", "mamba2_scan", "gated_rmsnorm",
