@@ -68,13 +68,14 @@ def sink_attention(h, w, p, m, eps, k, v):
     gate = torch.sigmoid(h @ _t(w, p + "g").T)           # (T, H)
     sink = _t(w, p + "sink")
     out = torch.zeros(T, H, dv, dtype=F)
+    hidden = torch.triu(torch.ones(T, T, dtype=torch.bool), diagonal=1)      # key j > query i
     for a in range(H):
         g = a // (H // G)
-        for i in range(T):
-            s = (k[:i + 1, g] @ q[i, a]) * m["scale"]
-            top = max(float(s.max()), float(sink[a]))
-            e = torch.exp(s - top)
-            out[i, a] = (e[:, None] * v[:i + 1, g]).sum(dim=0) / (e.sum() + math.exp(float(sink[a]) - top))
+        s = (q[:, a] @ k[:, g].T) * m["scale"]
+        s = s.masked_fill(hidden, float("-inf"))
+        top = torch.maximum(s.max(dim=-1).values, sink[a])
+        e = torch.exp(s - top[:, None])
+        out[:, a] = (e @ v[:, g]) / (e.sum(dim=-1) + torch.exp(sink[a] - top))[:, None]
     out = out * gate[:, :, None]
     return out.reshape(T, H * dv) @ _t(w, p + "o").T
 
@@ -154,3 +155,10 @@ def forward(config, w, tokens, streams=None):
         if streams is not None:
             streams.append(x.clone())
     return rms_norm(x, _t(w, "final.norm"), eps) @ _t(w, "embed").T
+
+
+def greedy(config, w, prompt, new_tokens):
+    tokens = list(prompt)
+    for _ in range(new_tokens):
+        tokens.append(int(forward(config, w, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
