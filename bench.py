@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
                     [--shape 8b|14b|32b|0.6b] [--prompt P] [--context C]
-                    [--workload decode|continuous|served|prefix|products|kodisun|surasun]
+                    [--workload decode|continuous|served|prefix|products|kodisun|surasun|dufinex]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -552,6 +552,147 @@ def surasun(args, sync):
     return 0
 
 
+DUFINEX_SHAPES = {
+    # (width, dense feed-forward inner size, experts, experts a token, layers as (mixer, reads the keys of, feed-forward))
+    "base": (2048, 6144, 32, 4, (("attention", None, "dense"), ("attention", 0, "moe"), ("channel_delta", None, "dense"),
+                                 ("attention", None, "moe"))),
+    "wide": (4096, 12288, 64, 8, (("channel_delta", None, "moe"), ("attention", None, "dense"))),
+}
+
+
+def dufinex_layers(W, ff, experts, top, kinds):
+    """Layers of real proportions: attention in heads of 128, four query heads a key head; the delta rule in
+    heads of 128 with values of 128, a key head per head, four taps; experts whose inner sizes add up, over a
+    token's choices, to the dense feed-forward's."""
+    mixers = {"attention": {"heads": W // 128, "kv_heads": W // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5},
+              "channel_delta": {"heads": W // 128, "kv_heads": W // 128, "dim": 128, "vdim": 128, "conv": 4}}
+    feeds = {"dense": {"kind": "dense", "ff": ff, "limit": 7.0},
+             "moe": {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff // top, "limit": 7.0}}}
+    listed = []
+    for kind, source, feed in kinds:
+        mixer = dict(mixers[kind])
+        if source is not None:
+            mixer["kv_from"] = source
+        listed.append({"type": kind, "mixer": mixer, "mlp": feeds[feed]})
+    return listed
+
+
+def dufinex(args, sync):
+    """Prefill and decode throughput of the Dufinex design at sizes that resemble a real model's layers
+    (random weights, a few layers, a vocabulary of 32,768), beside the Surasun design, the closest of the
+    others (softmax attention with a gate per head through the same kernels, recurrences with a state per
+    head), at the same width, layer count and feed-forward inner size, a layer of attention beside
+    retention where this one has attention and Mamba-2 where it has the delta rule. Both go through the
+    engine's own loop: one prompt in one step, then greedy decoding at batch 8 and 64 behind prompts of
+    1,024 tokens. `frac` prices a prompt's multiply-adds (the products with a token's share of the
+    experts, the recurrences' updates and reads, the attention's pairs) against the bfloat16 matrix peak,
+    and a decode step's bytes (the weights once, of the experts those a batch can reach, the states read
+    and written, the cached keys and values) against the HBM peak."""
+    import torch
+
+    from qwen3_from_scratch_amd.config.dufinex_config import DufinexConfig
+    from qwen3_from_scratch_amd.config.surasun_config import SurasunConfig
+    from qwen3_from_scratch_amd.engine import SyncEngine, random_model
+
+    vocab, prompt_len, decode_prompt, context = 32768, args.prefill_tokens, 1024, 4096
+    results = {}
+    for shape in ([args.dufinex_shape] if args.dufinex_shape != "all" else sorted(DUFINEX_SHAPES)):
+        W, ff, experts, top, kinds = DUFINEX_SHAPES[shape]
+        if args.layers:
+            kinds = tuple((k, None, f) for k, _, f in (kinds * args.layers)[:args.layers])
+        listed = dufinex_layers(W, ff, experts, top, kinds)
+        new = DufinexConfig.from_dict({"architecture": "Dufinex", "vocab": vocab, "width": W, "norm": {"eps": 1e-5},
+                                       "embedding": {"scale": 1.0}, "layers": listed})
+        other = SurasunConfig.from_dict({"architecture": "Surasun", "vocab": vocab, "width": W, "norm": {"eps": 1e-5},
+                                         "residual_mult": 1.0,
+                                         "layers": surasun_layers(W, ff, [("parallel" if k == "attention" else "mamba2", True)
+                                                                          for k, _, _ in kinds])})
+        for name, config in (("dufinex", new), ("surasun", other)):
+            if args.dufinex_only and name != args.dufinex_only:
+                continue
+            model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
+            gen = torch.Generator().manual_seed(1)
+            entry = {}
+            tensors = model.tensors()
+            # per token: matrix numbers every token meets, those of one expert's share, the recurrences' multiply-adds;
+            # per (query, key) pair; floats of state; cached numbers
+            matrices = sum(t[0] * t[1] for key, t in tensors.items()
+                           if len(t) == 2 and key != "embed" and ".hc" not in key and not key.endswith("conv") and ".mlp.e" not in key)
+            expert_numbers = sum(t[0] * t[1] for key, t in tensors.items() if ".mlp.e" in key)
+            scans = pairs_each = state = cached = 0
+            for layer in (listed if name == "dufinex" else config.to_dict()["layers"]):
+                m = layer["mixer"]
+                if layer["type"] == "channel_delta":
+                    scans += 4 * m["heads"] * m["dim"] * m["vdim"]
+                    state += m["heads"] * m["dim"] * m["vdim"] + 3 * (2 * m["kv_heads"] * m["dim"] + m["heads"] * m["vdim"])
+                elif layer["type"] == "attention":
+                    pairs_each += m["heads"] * (m["dim"] + m["vdim"])
+                    cached += 0 if m.get("kv_from") is not None else m["kv_heads"] * (m["dim"] + m["vdim"])
+                elif layer["type"] == "mamba2":
+                    scans += 3 * m["heads"] * m["state"] * m["vdim"]
+                    state += m["heads"] * m["state"] * m["vdim"] + 3 * (m["heads"] * m["vdim"] + 2 * m["state"])
+                else:
+                    scans += 3 * m["right"]["heads"] * m["right"]["dim"] * m["right"]["vdim"]
+                    state += m["right"]["heads"] * m["right"]["dim"] * m["right"]["vdim"]
+                    pairs_each += m["left"]["heads"] * (m["left"]["dim"] + m["left"]["vdim"])
+                    cached += m["left"]["kv_heads"] * (m["left"]["dim"] + m["left"]["vdim"])
+            share = top / experts
+            if "prefill" in args.phases:
+                room = prompt_len + 64
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=room, block_size=BLOCK,
+                                    num_blocks=-(-room // BLOCK), max_num_seqs=1, max_num_tokens=prompt_len,
+                                    chunked_prefill_size=prompt_len, enable_prefix_cache=False)
+                timings = []
+                for _ in range(4):
+                    engine.add_request(torch.randint(0, vocab, (prompt_len,), generator=gen).tolist(),
+                                       engine.default_params(1, temperature=0.0, ignore_eos=True))
+                    sync()
+                    t0 = time.perf_counter()
+                    engine.step()
+                    sync()
+                    timings.append(time.perf_counter() - t0)
+                    while engine.scheduler.has_work():
+                        engine.step()
+                seconds = sorted(timings[1:])[1]
+                flops = (2.0 * prompt_len * (matrices + share * expert_numbers + scans) + 2.0 * vocab * W
+                         + 2.0 * (prompt_len * (prompt_len + 1) / 2) * pairs_each)
+                entry["prefill"] = {"tokens": prompt_len, "tokens_per_s": round(prompt_len / seconds, 1),
+                                    "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+                del engine
+            for batch in ((8, 64) if "decode" in args.phases else ()):
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context,
+                                    block_size=BLOCK, num_blocks=batch * (context // BLOCK), max_num_seqs=batch,
+                                    max_num_tokens=max(2048, batch), chunked_prefill_size=2048, enable_prefix_cache=False)
+                params = engine.default_params(context - decode_prompt - 1, temperature=0.0, ignore_eos=True)
+                requests = [engine.add_request(torch.randint(0, vocab, (decode_prompt,), generator=gen).tolist(), params)
+                            for _ in range(batch)]
+                while any(r.is_prefill for r in requests) or len(engine.scheduler.waiting):
+                    engine.step()
+                for _ in range(args.warmup):
+                    engine.step()
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    engine.step()
+                sync()
+                step_s = (time.perf_counter() - t0) / args.steps
+                seen = decode_prompt + args.warmup + args.steps // 2
+                reached = min(1.0, batch * share)
+                need = 2 * (matrices + reached * expert_numbers + vocab * W) + batch * (8 * state + 2 * cached * seen)
+                entry["decode_b%d" % batch] = {"tokens_per_s": round(batch / step_s, 1), "ms_per_step": round(step_s * 1e3, 3),
+                                               "frac_hbm": round(need / step_s / PEAK_HBM, 4)}
+                del engine
+            results.setdefault(shape, {})[name] = entry
+            del model
+            torch.cuda.empty_cache()
+        results[shape]["sizes"] = {"width": W, "ff": ff, "experts": experts, "top": top, "vocab": vocab,
+                                   "layers": ["%s%s+%s" % (k, "" if src is None else "(keys of %d)" % src, f) for k, src, f in kinds]}
+    print(json.dumps({"metric": "Dufinex beside Surasun at equal size: prefill and decode tokens/s",
+                      "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+                      "steps": args.steps, "warmup": args.warmup, "shapes": results}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -563,17 +704,20 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products", "kodisun", "surasun"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products", "kodisun", "surasun", "dufinex"],
                     help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
                          "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused); "
                          "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off; "
                          "products: a layer's four products by the chosen kernel and by each tile shape of the "
-                         "hand-written one; kodisun, surasun: that design beside the dense decoder at equal size")
+                         "hand-written one; kodisun, surasun: that design beside the dense decoder at equal size; dufinex: "
+                         "that design beside Surasun at equal size")
     ap.add_argument("--kodisun-shape", default="all", choices=["all"] + sorted(KODISUN_SHAPES))
     ap.add_argument("--kodisun-only", default="", choices=["", "kodisun", "qwen3_dense"], help="one of the two models")
     ap.add_argument("--surasun-shape", default="all", choices=["all"] + sorted(SURASUN_SHAPES))
     ap.add_argument("--surasun-only", default="", choices=["", "surasun", "qwen3_dense"], help="one of the two models")
-    ap.add_argument("--phases", default="prefill,decode", help="of --workload kodisun or surasun: prefill, decode or both")
+    ap.add_argument("--dufinex-shape", default="all", choices=["all"] + sorted(DUFINEX_SHAPES))
+    ap.add_argument("--dufinex-only", default="", choices=["", "dufinex", "surasun"], help="one of the two models")
+    ap.add_argument("--phases", default="prefill,decode", help="of --workload kodisun, surasun or dufinex: prefill, decode or both")
     ap.add_argument("--single-copy", action="store_true",
                     help="hold the matrices once (no tile-ordered copy for steps of few rows): half the weights' memory, slower decoding")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
@@ -601,6 +745,10 @@ def main():
         torch.cuda.set_device(0)
         args.steps, args.warmup = min(args.steps, 32), min(args.warmup, 8)
         return surasun(args, torch.cuda.synchronize)
+    if args.workload == "dufinex":
+        torch.cuda.set_device(0)
+        args.steps, args.warmup = min(args.steps, 32), min(args.warmup, 8)
+        return dufinex(args, torch.cuda.synchronize)
     shape_name, raw = SHAPES[args.shape]
     raw = dict(raw)
     prompt_len, context = args.prompt, args.context
