@@ -22,12 +22,13 @@ __device__ inline float delta_sigmoid(float z) { return 1.f / (1.f + expf(-z)); 
 // and activations. `b_logits` (T, H) and `a_logits` (T, H dim), float32 rows possibly apart. Writes
 // `packed` (T, H, 3, DP) float32, per head [k | q | g], each padded with zeros to DP numbers (a
 // padded row of S then stays zero), q and k as unit vectors per head: x / sqrt(sum(x^2) + unit_eps),
-// q times dim^(-1/2), head h taking q and k of group h / (H / G); and `beta` (T, H).
+// q times dim^(-1/2), head h taking q and k of group h / (H / G); and `beta` (T, H, 2): beta itself and
+// the head's k . q, which the recurrence uses to read the current token's write without waiting for it.
 __global__ void __launch_bounds__(256) delta_prepare_kernel(
     const float* __restrict__ conv, const float* __restrict__ b_logits, long b_stride, const float* __restrict__ a_logits,
     long a_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log, float unit_eps,
     float* __restrict__ packed, float* __restrict__ beta, int H, int G, int dim, int vdim, int DP) {
-  extern __shared__ float unit[];             // (2, G, dim): q then k, finished
+  extern __shared__ float unit[];             // (2, G, dim): q then k, finished; then (G): k . q
   const int t = blockIdx.x;
   const int wave = threadIdx.x / Q3_WAVE, lane = threadIdx.x % Q3_WAVE, waves = blockDim.x / Q3_WAVE;
   const int C = 2 * G * dim + H * vdim;
@@ -39,6 +40,14 @@ __global__ void __launch_bounds__(256) delta_prepare_kernel(
     float r = rsqrtf(wave_sum(acc) + unit_eps);
     if (j < G) r *= rsqrtf((float)dim);
     for (int e = lane; e < dim; e += Q3_WAVE) unit[j * dim + e] = src[e] * r;
+  }
+  __syncthreads();
+  float* kq = unit + 2 * G * dim;
+  for (int j = wave; j < G; j += waves) {
+    float acc = 0.f;
+    for (int e = lane; e < dim; e += Q3_WAVE) acc += unit[j * dim + e] * unit[(G + j) * dim + e];
+    acc = wave_sum(acc);
+    if (lane == 0) kq[j] = acc;
   }
   __syncthreads();
   const int per = H / G;
@@ -57,7 +66,10 @@ __global__ void __launch_bounds__(256) delta_prepare_kernel(
     dst[DP + e] = q;
     dst[2 * DP + e] = g;
   }
-  for (int h = threadIdx.x; h < H; h += blockDim.x) beta[(size_t)t * H + h] = delta_sigmoid(b_logits[(size_t)t * b_stride + h]);
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    beta[((size_t)t * H + h) * 2] = delta_sigmoid(b_logits[(size_t)t * b_stride + h]);
+    beta[((size_t)t * H + h) * 2 + 1] = kq[h / per];
+  }
 }
 
 // ---- the recurrence ----
@@ -65,16 +77,6 @@ template <int CTRL>
 __device__ __forceinline__ float lanes_moved(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
-// The sum over a row of sixteen lanes, in all of them: neighbours, pairs of a quad, then the quads
-// rotated by four and by eight lanes, all in the vector unit's own lane crossing.
-__device__ __forceinline__ float row16_sum(float v) {
-  v += lanes_moved<0xB1>(v);      // quad_perm [1, 0, 3, 2]
-  v += lanes_moved<0x4E>(v);      // quad_perm [2, 3, 0, 1]
-  v += lanes_moved<0x124>(v);     // row_ror 4
-  v += lanes_moved<0x128>(v);     // row_ror 8
-  return v;
-}
-
 template <int R>
 __device__ __forceinline__ void load_run(const float* p, float (&v)[R]) {
   if constexpr (R >= 4) {
@@ -93,10 +95,19 @@ __device__ __forceinline__ void load_run(const float* p, float (&v)[R]) {
 // grid (H * ceil(vdim / 16), B), 256 threads: thread (column slot = t / 16, part = t % 16) keeps rows
 // part * R .. part * R + R - 1 of its column in registers. The tokens' [k | q | g] come `TC` tokens at
 // a time through shared memory, the next chunk's on their way (into registers) while this one is worked
-// on; per token and thread that is 4 R multiply-adds and two sums over sixteen lanes. The order of a
-// column's arithmetic does not depend on how the sequence was cut into steps or chunks. Results go
-// to `raw` (T, H vdim) float32; the division by the head's root mean square and the gate follow in
-// delta_finish_kernel.
+// on, and within a chunk the next token's numbers are read from shared memory while this token's are
+// worked on. A token's chain of dependent steps is what bounds the kernel (one wavefront a SIMD when a
+// single sequence is all there is), so the read-out does not wait for the write: with S' = diag(g) S,
+//   u = beta (v - S'^T k),   o = (S' + k u^T)^T q = S'^T q + u (k . q),
+// the two sums over the rows run side by side, k . q comes with the token, and the update S = S' + k u^T
+// is off the way to o. The order of a column's arithmetic does not depend on how the sequence was cut
+// into steps or chunks. Results go to `raw` (T, H vdim) float32; the division by the head's root mean
+// square and the gate follow in delta_finish_kernel.
+template <int R>
+struct DeltaToken {
+  float k[R], q[R], g[R], v, beta, kq;
+};
+
 template <int R, int TC>
 __global__ void __launch_bounds__(256) delta_scan_kernel(
     const float* __restrict__ packed, const float* __restrict__ beta, const float* __restrict__ conv,
@@ -108,7 +119,7 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
   constexpr int PF = (N4 + 255) / 256;              // pieces a thread brings
   __shared__ __attribute__((aligned(16))) float kqg[2][TC * ROW];
   __shared__ float sv[2][TC * Q3_DELTA_COLS];
-  __shared__ float sb[2][TC];
+  __shared__ __attribute__((aligned(8))) float sb[2][2 * TC];
   const int slices = (vdim + Q3_DELTA_COLS - 1) / Q3_DELTA_COLS;
   const int h = blockIdx.x / slices, c0 = (blockIdx.x % slices) * Q3_DELTA_COLS;
   const int b = blockIdx.y;
@@ -123,8 +134,14 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
 
   float* mine = state + (size_t)slots[b] * state_stride + ((size_t)h * vdim + (live ? c : 0)) * dim + part * R;
   float S[R];
+  // a thread's rows lie side by side in the state: 16-byte accesses where the column's start allows them
+  const bool whole = live && part * R + R <= dim && R >= 4 && ((size_t)mine % 16) == 0;
+  if (whole) {
+    load_run<R>(mine, S);
+  } else {
 #pragma unroll
-  for (int r = 0; r < R; ++r) S[r] = (live && part * R + r < dim) ? mine[r] : 0.f;
+    for (int r = 0; r < R; ++r) S[r] = (live && part * R + r < dim) ? mine[r] : 0.f;
+  }
 
   float4 ahead[PF];
   float ahead_v = 0.f, ahead_b = 0.f;
@@ -141,7 +158,7 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
       const int tok = tid >> 4, col = c0 + (tid & 15);
       ahead_v = (t0 + tok < end && col < vdim) ? conv[(size_t)(t0 + tok) * C + v_at + col] : 0.f;
     }
-    if (tid < TC) ahead_b = t0 + tid < end ? beta[(size_t)(t0 + tid) * H + h] : 0.f;
+    if (tid < 2 * TC) ahead_b = t0 + (tid >> 1) < end ? beta[((size_t)(t0 + (tid >> 1)) * H + h) * 2 + (tid & 1)] : 0.f;
   };
   auto put = [&](int buf) {
 #pragma unroll
@@ -150,7 +167,39 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
       if (at < N4) *reinterpret_cast<float4*>(&kqg[buf][4 * at]) = ahead[i];
     }
     if (tid < TC * Q3_DELTA_COLS) sv[buf][tid] = ahead_v;
-    if (tid < TC) sb[buf][tid] = ahead_b;
+    if (tid < 2 * TC) sb[buf][tid] = ahead_b;
+  };
+  auto read = [&](DeltaToken<R>& tok, int buf, int i) {      // token i of the chunk in `buf`, from shared memory
+    const float* row = &kqg[buf][i * ROW + part * R];
+    load_run<R>(row, tok.k);
+    load_run<R>(row + 2 * DP, tok.g);
+    load_run<R>(row + DP, tok.q);
+    tok.v = sv[buf][i * Q3_DELTA_COLS + slot];
+    const float2 bk = *reinterpret_cast<const float2*>(&sb[buf][2 * i]);
+    tok.beta = bk.x;
+    tok.kq = bk.y;
+  };
+  auto work = [&](const DeltaToken<R>& tok, int t) {
+    float seen[2] = {0.f, 0.f}, out[2] = {0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      S[r] *= tok.g[r];
+      seen[r & 1] += S[r] * tok.k[r];
+      out[r & 1] += S[r] * tok.q[r];
+    }
+    float a = seen[0] + seen[1], o = out[0] + out[1];
+    a += lanes_moved<0xB1>(a);      // quad_perm [1, 0, 3, 2]: the two sums over sixteen lanes, step by step side by side
+    o += lanes_moved<0xB1>(o);
+    a += lanes_moved<0x4E>(a);      // quad_perm [2, 3, 0, 1]
+    o += lanes_moved<0x4E>(o);
+    a += lanes_moved<0x124>(a);     // row_ror 4
+    o += lanes_moved<0x124>(o);
+    a += lanes_moved<0x128>(a);     // row_ror 8
+    o += lanes_moved<0x128>(o);
+    const float u = tok.beta * (tok.v - a);
+#pragma unroll
+    for (int r = 0; r < R; ++r) S[r] += tok.k[r] * u;
+    if (part == 0 && live) raw[(size_t)t * H * vdim + (size_t)h * vdim + c] = o + u * tok.kq;
   };
 
   fetch(start);
@@ -161,33 +210,33 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
     const bool more = t0 + TC < end;                // uniform in the block
     if (more) fetch(t0 + TC);
     const int n = end - t0 < TC ? end - t0 : TC;
-    for (int i = 0; i < n; ++i) {
-      const float* row = &kqg[buf][i * ROW + part * R];
-      float k[R], q[R], g[R];
-      load_run<R>(row, k);
-      load_run<R>(row + 2 * DP, g);
-      float seen = 0.f;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        S[r] *= g[r];
-        seen += S[r] * k[r];
+    // two tokens in work while the next two come from shared memory
+    DeltaToken<R> a0, a1, b0, b1;
+    auto at = [&](int i) { return i < TC ? i : TC - 1; };
+    read(a0, buf, 0);
+    read(a1, buf, at(1));
+    for (int i = 0; i < n; i += 4) {
+      read(b0, buf, at(i + 2));
+      read(b1, buf, at(i + 3));
+      work(a0, t0 + i);
+      if (i + 1 < n) work(a1, t0 + i + 1);
+      if (i + 2 < n) {
+        read(a0, buf, at(i + 4));
+        read(a1, buf, at(i + 5));
+        work(b0, t0 + i + 2);
+        if (i + 3 < n) work(b1, t0 + i + 3);
       }
-      seen = row16_sum(seen);
-      load_run<R>(row + DP, q);
-      const float u = sb[buf][i] * (sv[buf][i * Q3_DELTA_COLS + slot] - seen);
-      float o = 0.f;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        S[r] += k[r] * u;
-        o += S[r] * q[r];
-      }
-      o = row16_sum(o);
-      if (part == 0 && live) raw[(size_t)(t0 + i) * H * vdim + (size_t)h * vdim + c] = o;
     }
     if (more) put(buf ^ 1);
     __syncthreads();
   }
-  if (live) {
+  if (whole) {
+    if constexpr (R >= 4) {
+#pragma unroll
+      for (int j = 0; j < R / 4; ++j)
+        *reinterpret_cast<float4*>(mine + 4 * j) = make_float4(S[4 * j], S[4 * j + 1], S[4 * j + 2], S[4 * j + 3]);
+    }
+  } else if (live) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
       if (part * R + r < dim) mine[r] = S[r];
@@ -212,12 +261,12 @@ __global__ void delta_finish_kernel(const float* __restrict__ raw, const float* 
 }
 
 // The padded key size the recurrence works with, and the floats of scratch a step of T tokens needs:
-// packed (T, H, 3, DP), beta (T, H), raw (T, H vdim).
+// packed (T, H, 3, DP), beta (T, H, 2), raw (T, H vdim).
 extern "C" int q3_channel_delta_padded(int dim) {
   return dim <= 32 ? 32 : (dim <= 64 ? 64 : (dim <= 128 ? 128 : 256));
 }
 extern "C" long q3_channel_delta_workspace(int T, int H, int dim, int vdim) {
-  return (long)T * H * (3 * q3_channel_delta_padded(dim) + 1 + vdim);
+  return (long)T * H * (3 * q3_channel_delta_padded(dim) + 2 + vdim);
 }
 
 // conv float32 (T, 2 G dim + H vdim) contiguous; b_logits (T, H), a_logits (T, H dim) and gate (T, H vdim)
@@ -236,17 +285,20 @@ extern "C" int q3_channel_delta(const float* conv, const float* b_logits, long b
   const int DP = q3_channel_delta_padded(dim);
   float* packed = work;
   float* beta = packed + (size_t)T * H * 3 * DP;
-  float* raw = beta + (size_t)T * H;
-  hipLaunchKernelGGL(delta_prepare_kernel, dim3(T), dim3(256), (size_t)2 * G * dim * sizeof(float), stream, conv, b_logits,
+  float* raw = beta + (size_t)T * H * 2;
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3(T), dim3(256), ((size_t)2 * G * dim + G) * sizeof(float), stream, conv, b_logits,
                      b_stride, a_logits, a_stride, dt_bias, a_log, unit_eps, packed, beta, H, G, dim, vdim, DP);
   const dim3 grid(H * slices, B);
 #define Q3_DELTA(RR, TT)                                                                                             \
   hipLaunchKernelGGL((delta_scan_kernel<RR, TT>), grid, dim3(256), 0, stream, packed, beta, conv, state, state_stride, \
                      slots, cu, raw, H, G, dim, vdim)
-  if (DP == 32) Q3_DELTA(2, 16);
-  else if (DP == 64) Q3_DELTA(4, 16);
-  else if (DP == 128) Q3_DELTA(8, 16);
-  else Q3_DELTA(16, 8);
+  // steps of a token or two a sequence (decoding): chunks of two tokens, whose few kilobytes of shared memory let
+  // a CU hold as many blocks as its threads allow, where the wait for each block's state is what counts
+  const bool few = T <= 2 * B;
+  if (DP == 32) { if (few) Q3_DELTA(2, 2); else Q3_DELTA(2, 16); }
+  else if (DP == 64) { if (few) Q3_DELTA(4, 2); else Q3_DELTA(4, 16); }
+  else if (DP == 128) { if (few) Q3_DELTA(8, 2); else Q3_DELTA(8, 16); }
+  else { if (few) Q3_DELTA(16, 2); else Q3_DELTA(16, 8); }
 #undef Q3_DELTA
   const int threads = vdim >= 256 ? 256 : (vdim >= 128 ? 128 : 64);
   Q3_DISPATCH_DTYPE(act_dtype, TA, hipLaunchKernelGGL(delta_finish_kernel<TA>, dim3(T, H), dim3(threads), 0, stream, raw,
