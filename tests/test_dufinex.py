@@ -429,6 +429,26 @@ def test_one_part_alone(tmp_path, kind, dtype):
     _all_cuttings(folder, requests, want, dtype, "cuda", 16)
 
 
+ONES = _model(61, 32, [_layer(_delta(4, 2, 12, 10, 1)), _layer(_delta(2, 1, 8, 10, 3), _moe(1, 1, 8))])
+
+
+def test_sizes_of_one_on_the_host(cpu_ops, tmp_path):
+    """A convolution of one tap (no tail in the state), one expert, and a model without attention (no pages at all)."""
+    folder = _write(tmp_path / "m", ONES)
+    requests = _requests(folder, lengths=(20, 3, 1))
+    _, _, want = _truth(folder, requests)
+    _all_cuttings(folder, requests, want, "float32", "cpu", 8)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_of_one(tmp_path, dtype):
+    folder = _write(tmp_path / "m", ONES, **(dict(peak=2.0) if dtype == "float32" else dict(std=0.06)))
+    requests = _requests(folder, lengths=(45, 3, 1, 100))
+    _, _, want = _truth(folder, requests)
+    _all_cuttings(folder, requests, want, dtype, "cuda", 16)
+
+
 @pytest.mark.gpu
 def test_stream_behind_every_layer(tmp_path):
     folder = _write(tmp_path / "m", WIDE)

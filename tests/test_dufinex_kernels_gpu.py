@@ -124,6 +124,7 @@ ATTENTION_CASES = [
     (torch.bfloat16, 8, 2, 128, 128, 16, [(300, 3000), (1, 50), (2, 9)]),       # a portion over many keys, split
     (torch.bfloat16, 4, 4, 64, 64, 32, [(600, 600)]),
     (torch.bfloat16, 4, 2, 32, 64, 16, [(7, 40), (1, 33)]),                    # key and value sizes differ: the general kernel
+    (torch.bfloat16, 16, 1, 64, 64, 16, [(3, 40), (1, 33), (1, 900)]),          # as many heads on a key head as a block of rows
     (torch.bfloat16, 32, 1, 64, 64, 16, [(3, 40), (1, 33)]),                   # more heads on a key head than a block of rows
 ]
 
