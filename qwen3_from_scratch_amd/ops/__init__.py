@@ -590,17 +590,10 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
     # (with inner sizes in steps of 64: tiles of 256 by the dense path's copies and stages)
     many = 3 if width % 64 == 0 and ff % 64 == 0 else 2
     tile_rows = lib.q3_moe_tile_rows((many if P >= 96 * E else 1) if cores else 0)
-    max_tiles = -(-P // tile_rows) + E
-    book = torch.empty((E + 1 + 2 * P + 2 * max_tiles + 1,), dtype=torch.int32, device=h.device)
-    offsets, pair_of_slot, slot_of_pair = book[:E + 1], book[E + 1:E + 1 + P], book[E + 1 + P:E + 1 + 2 * P]
-    at = E + 1 + 2 * P
-    tile_expert, tile_first, n_tiles = book[at:at + max_tiles], book[at + max_tiles:at + 2 * max_tiles], book[at + 2 * max_tiles:]
+    tiles, pair_of_slot, slot_of_pair = _moe_book(lib, chosen, E, tile_rows)
     stream = _stream()
-    _check(lib.q3_moe_align(_ptr(chosen), P, E, tile_rows, _ptr(offsets), _ptr(pair_of_slot), _ptr(slot_of_pair),
-                            _ptr(tile_expert), _ptr(tile_first), _ptr(n_tiles), stream), "moe_align")
     hidden = torch.empty((P, ff), dtype=h.dtype, device=h.device)
     y = torch.empty((P, width), dtype=h.dtype, device=h.device)
-    tiles = (_ptr(tile_expert), _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles)
     if cores:
         _check(lib.q3_moe_linear_mma(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(up), _ptr(hidden), *tiles, ff, width,
                                      GELU_KINDS[activation], tile_rows, stream), "moe_linear")
