@@ -64,7 +64,8 @@ def test_glu_clamped(dtype, T, I):
 
 @pytest.mark.parametrize("dtype,W,ff,E,top,T", [
     (torch.float32, 48, 40, 6, 2, 29), (torch.float32, 40, 10, 3, 3, 7), (torch.bfloat16, 64, 96, 16, 1, 300),
-    (torch.bfloat16, 128, 64, 8, 3, 2000), (torch.bfloat16, 64, 32, 4, 2, 5), (torch.bfloat16, 48, 24, 70, 4, 130)])
+    (torch.bfloat16, 128, 64, 8, 3, 2000), (torch.bfloat16, 64, 32, 4, 2, 5), (torch.bfloat16, 48, 24, 70, 4, 130),
+    (torch.bfloat16, 160, 96, 8, 2, 1500), (torch.float32, 160, 96, 8, 2, 1500)])
 def test_experts_by_sigmoid_scores(dtype, W, ff, E, top, T):
     g = _gen(W + E + T)
     h = _rand(g, T, W, dtype=dtype)
