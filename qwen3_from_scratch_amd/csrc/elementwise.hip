@@ -1,4 +1,4 @@
-// Embedding row gather and the SwiGLU activation.
+// Embedding row gather and the gated activations (SwiGLU and its gelu forms).
 #include "common.h"
 
 // out[t, :] = float(table[ids[t], :]) * scale. An id outside the table gives a row of
@@ -15,10 +15,18 @@ __global__ void embed_rows_kernel(const int* __restrict__ ids, const T* __restri
   for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ok ? to_float(row[j]) * scale : 0.f;
 }
 
-// out[t, j] = silu(gate[t, j]) * up[t, j] for rows that interleave the two:
-// gate_up[t, 2j] = gate[t, j], gate_up[t, 2j + 1] = up[t, j].
-// silu(g) = g / (1 + exp(-g)), evaluated in float32 and rounded once.
-template <typename T>
+// out[t, j] = act(gate[t, j]) * up[t, j] for rows that interleave the two:
+// gate_up[t, 2j] = gate[t, j], gate_up[t, 2j + 1] = up[t, j]. ACT 0: silu(g) = g / (1 + exp(-g));
+// 1: the tanh form of gelu, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))); 2: the exact gelu,
+// 0.5 g (1 + erf(g / sqrt 2)). Evaluated in float32 and rounded once.
+template <int ACT>
+__device__ inline float gate_value(float g) {
+  if (ACT == 0) return g / (1.f + expf(-g));
+  if (ACT == 1) return 0.5f * g * (1.f + tanhf(0.79788456080286536f * (g + 0.044715f * g * g * g)));
+  return 0.5f * g * (1.f + erff(g * 0.70710678118654752f));
+}
+
+template <typename T, int ACT>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int I) {
   const int t = blockIdx.y;
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
@@ -26,10 +34,11 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
   const T* row = gate_up + (size_t)t * 2 * I;
   const float g = to_float(row[2 * j]);
   const float u = to_float(row[2 * j + 1]);
-  out[(size_t)t * I + j] = from_float<T>(g / (1.f + expf(-g)) * u);
+  out[(size_t)t * I + j] = from_float<T>(gate_value<ACT>(g) * u);
 }
 
 // The same, eight outputs per thread with 16-byte loads and stores; bfloat16, I a multiple of 8.
+template <int ACT>
 __global__ void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int I) {
   const int t = blockIdx.y;
   const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
@@ -44,8 +53,8 @@ __global__ void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* _
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const float g0 = bf16_to_float(a.e[2 * i]), g1 = bf16_to_float(b.e[2 * i]);
-    o.e[i] = float_to_bf16(g0 / (1.f + expf(-g0)) * bf16_to_float(a.e[2 * i + 1]));
-    o.e[4 + i] = float_to_bf16(g1 / (1.f + expf(-g1)) * bf16_to_float(b.e[2 * i + 1]));
+    o.e[i] = float_to_bf16(gate_value<ACT>(g0) * bf16_to_float(a.e[2 * i + 1]));
+    o.e[4 + i] = float_to_bf16(gate_value<ACT>(g1) * bf16_to_float(b.e[2 * i + 1]));
   }
   *reinterpret_cast<uint4*>(out + (size_t)t * I + j) = o.u;
 }
@@ -95,8 +104,8 @@ extern "C" int q3_embed_rows(const int* ids, const void* table, float* out, int 
   return q3_launch_status();
 }
 
-extern "C" int q3_swiglu(const void* gate_up, void* out, int T, int I, int dtype, hipStream_t stream) {
-  if (T <= 0 || I <= 0 || T > 65535 * 32) return Q3_ERR_BAD_ARGUMENT;
+template <int ACT>
+static int launch_gated_act(const void* gate_up, void* out, int T, int I, int dtype, hipStream_t stream) {
   const int threads = 256;
   // blockIdx.y carries the row; rows beyond 65535 are covered by several launches
   for (int t0 = 0; t0 < T; t0 += 65535) {
@@ -104,16 +113,28 @@ extern "C" int q3_swiglu(const void* gate_up, void* out, int T, int I, int dtype
     if (dtype == Q3_BF16 && I % 8 == 0) {
       const int per_row = I / 8;
       const int vt = per_row >= 256 ? 256 : 64;
-      hipLaunchKernelGGL(swiglu_vec8_kernel, dim3((per_row + vt - 1) / vt, rows), dim3(vt), 0, stream,
+      hipLaunchKernelGGL(swiglu_vec8_kernel<ACT>, dim3((per_row + vt - 1) / vt, rows), dim3(vt), 0, stream,
                          (const bf16_t*)gate_up + (size_t)t0 * 2 * I, (bf16_t*)out + (size_t)t0 * I, I);
       continue;
     }
     Q3_DISPATCH_DTYPE(dtype, TT,
-                      hipLaunchKernelGGL(swiglu_kernel<TT>, dim3((I + threads - 1) / threads, rows),
+                      hipLaunchKernelGGL((swiglu_kernel<TT, ACT>), dim3((I + threads - 1) / threads, rows),
                                          dim3(threads), 0, stream,
                                          (const TT*)gate_up + (size_t)t0 * 2 * I, (TT*)out + (size_t)t0 * I, I));
   }
   return q3_launch_status();
+}
+
+// `act`: 0 silu, 1 the tanh form of gelu, 2 the exact gelu.
+extern "C" int q3_gated_act(const void* gate_up, void* out, int T, int I, int act, int dtype, hipStream_t stream) {
+  if (T <= 0 || I <= 0 || T > 65535 * 32 || act < 0 || act > 2) return Q3_ERR_BAD_ARGUMENT;
+  if (act == 0) return launch_gated_act<0>(gate_up, out, T, I, dtype, stream);
+  if (act == 1) return launch_gated_act<1>(gate_up, out, T, I, dtype, stream);
+  return launch_gated_act<2>(gate_up, out, T, I, dtype, stream);
+}
+
+extern "C" int q3_swiglu(const void* gate_up, void* out, int T, int I, int dtype, hipStream_t stream) {
+  return q3_gated_act(gate_up, out, T, I, 0, dtype, stream);
 }
 
 // out = gelu(x), elementwise in float32, rounded once: kind 0 the exact form

@@ -13,7 +13,9 @@
 #include <math.h>
 
 // ---------------------------------------------------------------------------
-// One block per token. `down` (T, q_rank + kv_rank + rot_dim) is the joint down-projection.
+// One block per token. `down` (T, q_rank + kv_rank + rot_dim) is the joint down-projection; its rows
+// lie `down_stride` numbers apart (a wider product may carry further columns behind these), and
+// rot_dim may be 0 (keys without a rotated part).
 //   cq[t]    = rms_norm(down[t, :q_rank]) * q_weight                       -> (T, q_rank)
 //   cache row of (sequence, position) = [rms_norm(down[t, q_rank:q_rank+kv_rank]) * kv_weight |
 //                                        rotate(down[t, q_rank+kv_rank:])]
@@ -21,7 +23,7 @@
 // (a float32 product), with cos and sin multiplied by rot_factor; numbers beyond 2 rot_pairs pass.
 // ---------------------------------------------------------------------------
 template <typename T, typename W>
-__global__ void latent_prepare_kernel(const T* __restrict__ down, int q_rank, int kv_rank, int rot_dim,
+__global__ void latent_prepare_kernel(const T* __restrict__ down, long down_stride, int q_rank, int kv_rank, int rot_dim,
                                       const W* __restrict__ q_weight, const W* __restrict__ kv_weight, float eps,
                                       const float* __restrict__ inv_freq, int rot_pairs, float rot_factor,
                                       const int* __restrict__ positions, const int* __restrict__ seq_index,
@@ -32,7 +34,7 @@ __global__ void latent_prepare_kernel(const T* __restrict__ down, int q_rank, in
   float* row = smem + 32;
   const int t = blockIdx.x;
   const int R = q_rank + kv_rank + rot_dim;
-  const T* src = down + (size_t)t * R;
+  const T* src = down + (size_t)t * down_stride;
   float acc_q = 0.f, acc_kv = 0.f;
   for (int j = threadIdx.x; j < R; j += blockDim.x) {
     const float v = to_float(src[j]);
@@ -205,7 +207,10 @@ __global__ void rotate_heads_kernel(const T* __restrict__ x, long x_row, int x_h
 // at once, so a tile is loaded once. Tiles start at absolute positions that are multiples of 32,
 // so the order in which a row's sums are formed does not depend on how the sequence was cut into
 // steps or on what else the block serves. Row of token i (position p = kv_len - q_len + i) sees
-// positions j <= p, and with a window w > 0 only p - j < w.
+// positions j <= p, and with a window w > 0 only p - j < w. With `sink` (H floats) the softmax's
+// denominator of head h also holds exp(sink[h]), a term without a key and a value that is not
+// scaled; with `gate` (rows `gate_stride` apart, H numbers each) head h's result is multiplied by
+// sigmoid(gate[token, h]).
 // ---------------------------------------------------------------------------
 #define LAT_BM 16
 #define LAT_BN 32
@@ -216,7 +221,9 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const T* __restrict__ 
                                                           const int* __restrict__ block_table, int bt_stride,
                                                           const int* __restrict__ cu_q,
                                                           const int* __restrict__ kv_lens, int H, int Dk, int Dv,
-                                                          int page, float scale, int window) {
+                                                          int page, float scale, int window,
+                                                          const float* __restrict__ sink, const T* __restrict__ gate,
+                                                          long gate_stride) {
   extern __shared__ float smem[];
   const int b = blockIdx.y;
   const int q0 = cu_q[b];
@@ -310,7 +317,9 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const T* __restrict__ 
     }
   }
   if (my_row) {
-    const float inv = 1.f / l_run;
+    if (sink) l_run += expf(sink[my_head] - m_run);
+    float inv = 1.f / l_run;
+    if (gate) inv /= 1.f + expf(-to_float(gate[(size_t)(q0 + my_tok) * gate_stride + my_head]));
     T* o = out + ((size_t)(q0 + my_tok) * H + my_head) * Dv;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -365,6 +374,7 @@ __device__ inline bool lma_find_tile(const int* __restrict__ cu_q, int B, int H,
 // block walks its share of the tiles and leaves float32 sums that are not yet divided, with the
 // row's maximum (in the exponent's units) and sum, in `partial` ((rows, splits, Dv + 2) floats,
 // rows numbered (packed token, head)); `latent_attn_merge_kernel` joins the shares in their order.
+// `sink` and `gate` as in the general kernel; with shares they join in the merge.
 template <int KS, int NV, int HALVES>
 __global__ __launch_bounds__(256 * HALVES) void latent_attn_mma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                                                               const bf16_t* __restrict__ cache, int num_pages,
@@ -372,7 +382,9 @@ __global__ __launch_bounds__(256 * HALVES) void latent_attn_mma_kernel(const bf1
                                                               const int* __restrict__ cu_q,
                                                               const int* __restrict__ kv_lens, int B, int H, int Dk,
                                                               int Dv, int page, float scale_log2, int window,
-                                                              int splits, float* __restrict__ partial) {
+                                                              int splits, float* __restrict__ partial,
+                                                              const float* __restrict__ sink,
+                                                              const bf16_t* __restrict__ gate, long gate_stride) {
   extern __shared__ __align__(16) unsigned char lma_smem[];
   int b, m0;
   if (!lma_find_tile(cu_q, B, H, blockIdx.x, b, m0)) return;
@@ -577,7 +589,10 @@ __global__ __launch_bounds__(256 * HALVES) void latent_attn_mma_kernel(const bf1
     }
     return;
   }
-  const float inv = 1.f / l_run;
+  // the sink joins where the row's sum is final: exp(sink) against the exponent's reference
+  if (sink) l_run += __builtin_amdgcn_exp2f(fmaf(sink[head], 1.44269504088896341f, -m_run));
+  float inv = 1.f / l_run;
+  if (gate) inv /= 1.f + expf(-bf16_to_float(gate[(size_t)(q0 + tok) * gate_stride + head]));
   bf16_t* o = out + ((size_t)(q0 + tok) * H + head) * Dv + 4 * grp;
 #pragma unroll
   for (int nb = 0; nb < NV; ++nb) {
@@ -593,8 +608,11 @@ __global__ __launch_bounds__(256 * HALVES) void latent_attn_mma_kernel(const bf1
   }
 }
 
-// out[row] = sum_s 2^(m_s - m) acc_s / sum_s 2^(m_s - m) l_s, m = max_s m_s, the shares in their order.
-__global__ void latent_attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out, int Dv, int splits) {
+// out[row] = sum_s 2^(m_s - m) acc_s / sum_s 2^(m_s - m) l_s, m = max_s m_s, the shares in their order;
+// the sink's term joins the denominator and the gate multiplies the quotient, as in the kernels above.
+__global__ void latent_attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out, int Dv, int splits,
+                                         int H, const float* __restrict__ sink, const bf16_t* __restrict__ gate,
+                                         long gate_stride) {
   const size_t row = blockIdx.x;
   const float* src = partial + row * splits * (Dv + 2);
   float m = -INFINITY;
@@ -604,7 +622,9 @@ __global__ void latent_attn_merge_kernel(const float* __restrict__ partial, bf16
     const float ms = src[(size_t)s * (Dv + 2) + Dv];
     if (ms > -INFINITY) l += exp2f(ms - m) * src[(size_t)s * (Dv + 2) + Dv + 1];
   }
-  const float inv = 1.f / l;
+  if (sink) l += exp2f(sink[row % H] * 1.44269504088896341f - m);
+  float inv = 1.f / l;
+  if (gate) inv /= 1.f + expf(-bf16_to_float(gate[(row / H) * gate_stride + row % H]));
   for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
     float a = 0.f;
     for (int s = 0; s < splits; ++s) {
@@ -621,13 +641,14 @@ static int raise_shared_memory(const void* kernel, size_t smem) {
   return (int)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
 }
 
-extern "C" int q3_latent_prepare(const void* down, int T, int q_rank, int kv_rank, int rot_dim, const void* q_weight,
+extern "C" int q3_latent_prepare(const void* down, long down_stride, int T, int q_rank, int kv_rank, int rot_dim, const void* q_weight,
                                  const void* kv_weight, int w_dtype, float eps, const float* inv_freq, int rot_pairs,
                                  float rot_factor, const int* positions, const int* seq_index,
                                  const int* block_table, int bt_stride, int bt_rows, void* cache, int page,
                                  int num_pages, void* cq, int dtype, hipStream_t stream) {
-  if (T <= 0 || q_rank <= 0 || kv_rank <= 0 || rot_dim <= 0 || 2 * rot_pairs > rot_dim || rot_pairs < 0)
+  if (T <= 0 || q_rank <= 0 || kv_rank <= 0 || rot_dim < 0 || 2 * rot_pairs > rot_dim || rot_pairs < 0)
     return Q3_ERR_BAD_ARGUMENT;
+  if (down_stride < q_rank + kv_rank + rot_dim || (rot_pairs > 0 && !inv_freq)) return Q3_ERR_BAD_ARGUMENT;
   if (cache && (!block_table || page <= 0 || num_pages <= 0 || bt_stride <= 0)) return Q3_ERR_BAD_ARGUMENT;
   const int R = q_rank + kv_rank + rot_dim;
   const size_t smem = (size_t)(32 + R) * sizeof(float);
@@ -636,8 +657,8 @@ extern "C" int q3_latent_prepare(const void* down, int T, int q_rank, int kv_ran
   Q3_DISPATCH_DTYPE(dtype, TT, Q3_DISPATCH_DTYPE(w_dtype, WW, {
     int e = raise_shared_memory((const void*)latent_prepare_kernel<TT, WW>, smem);
     if (e) return e;
-    hipLaunchKernelGGL((latent_prepare_kernel<TT, WW>), dim3(T), dim3(threads), smem, stream, (const TT*)down, q_rank,
-                       kv_rank, rot_dim, (const WW*)q_weight, (const WW*)kv_weight, eps, inv_freq, rot_pairs,
+    hipLaunchKernelGGL((latent_prepare_kernel<TT, WW>), dim3(T), dim3(threads), smem, stream, (const TT*)down, down_stride,
+                       q_rank, kv_rank, rot_dim, (const WW*)q_weight, (const WW*)kv_weight, eps, inv_freq, rot_pairs,
                        rot_factor, positions, seq_index, block_table, bt_stride, bt_rows, (TT*)cache, page, num_pages,
                        (TT*)cq);
     return q3_launch_status();
@@ -693,7 +714,8 @@ extern "C" int q3_rotate_heads(const void* x, long x_row, int x_head, void* out,
 template <typename T, int NV>
 static int launch_latent_attn(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
                               int bt_stride, const int* cu_q, const int* kv_lens, int B, int H, int Dk, int Dv,
-                              int page, float scale, int window, int max_q_len, hipStream_t stream) {
+                              int page, float scale, int window, int max_q_len, const float* sink, const void* gate,
+                              long gate_stride, hipStream_t stream) {
   const size_t smem = (size_t)(LAT_BM * Dk + LAT_BN * (Dk + 1) + LAT_BM * (LAT_BN + 1)) * sizeof(float);
   int e = raise_shared_memory((const void*)latent_attn_kernel<T, NV>, smem);
   if (e) return e;
@@ -701,7 +723,7 @@ static int launch_latent_attn(const void* q, void* out, const void* cache, int n
   if (tiles > 0x7fffffffL || B > 65535) return Q3_ERR_UNSUPPORTED;
   hipLaunchKernelGGL((latent_attn_kernel<T, NV>), dim3((unsigned)tiles, B), dim3(256), smem, stream, (const T*)q,
                      (T*)out, (const T*)cache, num_pages, block_table, bt_stride, cu_q, kv_lens, H, Dk, Dv, page, scale,
-                     window);
+                     window, sink, (const T*)gate, gate_stride);
   return q3_launch_status();
 }
 
@@ -709,7 +731,7 @@ template <int KS, int NV, int HALVES>
 static int launch_latent_attn_mma(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
                                   int bt_stride, const int* cu_q, const int* kv_lens, int B, int T, int H, int Dk,
                                   int Dv, int page, float scale, int window, int splits, float* partial,
-                                  hipStream_t stream) {
+                                  const float* sink, const void* gate, long gate_stride, hipStream_t stream) {
   const size_t smem = (size_t)(LMA_BN * (Dk + LMA_KPAD) + Dv * LMA_VLD) * sizeof(bf16_t);
   int e = raise_shared_memory((const void*)latent_attn_mma_kernel<KS, NV, HALVES>, smem);
   if (e) return e;
@@ -717,10 +739,11 @@ static int launch_latent_attn_mma(const void* q, void* out, const void* cache, i
   if (tiles > 0x7fffffffL || splits < 1 || splits > 65535 || (splits > 1 && !partial)) return Q3_ERR_UNSUPPORTED;
   hipLaunchKernelGGL((latent_attn_mma_kernel<KS, NV, HALVES>), dim3((unsigned)tiles, splits), dim3(256 * HALVES), smem, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, num_pages, block_table, bt_stride, cu_q,
-                     kv_lens, B, H, Dk, Dv, page, scale * 1.44269504088896341f, window, splits, partial);
+                     kv_lens, B, H, Dk, Dv, page, scale * 1.44269504088896341f, window, splits, partial, sink,
+                     (const bf16_t*)gate, gate_stride);
   if (splits > 1)
     hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)((long)T * H)), dim3(Dv >= 256 ? 256 : 64), 0, stream,
-                       partial, (bf16_t*)out, Dv, splits);
+                       partial, (bf16_t*)out, Dv, splits, H, sink, (const bf16_t*)gate, gate_stride);
   return q3_launch_status();
 }
 
@@ -732,32 +755,34 @@ extern "C" int q3_latent_attention_fast_path(int Dk, int Dv, int dtype) {
 extern "C" int q3_latent_attention(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
                                    int bt_stride, const int* cu_q, const int* kv_lens, int B, int T, int H, int Dk,
                                    int Dv, int page, float scale, int window, int max_q_len, int dtype, int general,
-                                   int splits, float* partial, hipStream_t stream) {
+                                   int splits, float* partial, const float* sink, const void* gate, long gate_stride,
+                                   hipStream_t stream) {
   if (B <= 0 || T <= 0 || H <= 0 || Dk <= 0 || Dv <= 0 || Dv > Dk || page <= 0 || max_q_len <= 0 || window < 0)
     return Q3_ERR_BAD_ARGUMENT;
   if (Dv > 1024) return Q3_ERR_UNSUPPORTED;
+  if (gate && gate_stride < H) return Q3_ERR_BAD_ARGUMENT;
   if (!general && q3_latent_attention_fast_path(Dk, Dv, dtype)) {
     if (Dk <= 192 && Dv <= 128)
       return launch_latent_attn_mma<6, 8, 1>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
-                                          Dv, page, scale, window, splits, partial, stream);
+                                          Dv, page, scale, window, splits, partial, sink, gate, gate_stride, stream);
     if (Dk <= 320 && Dv <= 256)
       return launch_latent_attn_mma<10, 16, 1>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H,
-                                            Dk, Dv, page, scale, window, splits, partial, stream);
+                                            Dk, Dv, page, scale, window, splits, partial, sink, gate, gate_stride, stream);
     return launch_latent_attn_mma<18, 16, 2>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
-                                          Dv, page, scale, window, splits, partial, stream);
+                                          Dv, page, scale, window, splits, partial, sink, gate, gate_stride, stream);
   }
   Q3_DISPATCH_DTYPE(dtype, TT, {
     if (Dv <= 128)
       return launch_latent_attn<TT, 8>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
-                                       page, scale, window, max_q_len, stream);
+                                       page, scale, window, max_q_len, sink, gate, gate_stride, stream);
     if (Dv <= 256)
       return launch_latent_attn<TT, 16>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
-                                        page, scale, window, max_q_len, stream);
+                                        page, scale, window, max_q_len, sink, gate, gate_stride, stream);
     if (Dv <= 512)
       return launch_latent_attn<TT, 32>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
-                                        page, scale, window, max_q_len, stream);
+                                        page, scale, window, max_q_len, sink, gate, gate_stride, stream);
     return launch_latent_attn<TT, 64>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
-                                      page, scale, window, max_q_len, stream);
+                                      page, scale, window, max_q_len, sink, gate, gate_stride, stream);
   });
   return Q3_ERR_BAD_ARGUMENT;
 }

@@ -12,23 +12,29 @@ __device__ inline float moe_gelu(float z, int kind) {
 }
 
 // ---------------------------------------------------------------------------
-// The router's choice. One wavefront per token, from its float32 logits z (E numbers). `mode` 0:
-// s = softmax(z) over all E experts, then `top` times the largest remaining score (the lowest
-// index among equals); weight_k = s_k / (sum of the chosen s + 1e-20). `mode` 1: s = sigmoid(z), each
-// expert for itself; the `top` largest are those with the largest z (chosen by z, which still tells
-// experts apart where the sigmoid has run into 1); weight_k = s_k as it is. Every lane holds every
-// reduced number and writes the same value to the same place of shared memory, so nothing here
-// waits for another lane's write.
+// The router's choice. One wavefront per token, from its float32 logits z (E numbers, a token's
+// `row_stride` apart). `mode` 0: s = softmax(z) over all E experts, then `top` times the largest
+// remaining score (the lowest index among equals); weight_k = s_k / (sum of the chosen s + 1e-20).
+// `mode` 1: s = sigmoid(z), each expert for itself; the `top` largest are those with the largest z
+// (chosen by z, which still tells experts apart where the sigmoid has run into 1); weight_k = s_k as it
+// is. `mode` 2: s = sigmoid(z); the choice goes by c = s + correction[e] and only among the experts of
+// `keep` of the `groups` equal groups of neighbours, those whose two largest c sum highest (the lowest
+// group among equals; the others' c count as minus infinity); weight_k = s_k as it is, without the
+// correction. Every lane holds every reduced number; what one lane writes to shared memory and
+// another reads is separated by the wavefront's barrier.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__ logits, int n_tokens, int E, int top,
-                                                       int mode, int* __restrict__ chosen, float* __restrict__ weights) {
+__global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__ logits, long row_stride, int n_tokens,
+                                                       int E, int top, int mode, const float* __restrict__ correction,
+                                                       int groups, int keep, int* __restrict__ chosen,
+                                                       float* __restrict__ weights) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x / Q3_WAVE, lane = threadIdx.x % Q3_WAVE;
   const int t = blockIdx.x * (blockDim.x / Q3_WAVE) + wave;
   if (t >= n_tokens) return;
-  float* z = smem + (size_t)wave * (E + top);     // the wavefront's scores, then the chosen ones
+  float* z = smem + (size_t)wave * (E + top + groups);     // the wavefront's scores, then the chosen ones, then the groups'
   float* picked = z + E;
-  const float* src = logits + (size_t)t * E;
+  float* group_score = picked + top;
+  const float* src = logits + (size_t)t * row_stride;
   float total = 1.f;
   if (mode == 0) {
     float biggest = -INFINITY;
@@ -41,10 +47,55 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
       total += p;
     }
     total = wave_sum(total);
-  } else {
+  } else if (mode == 1) {
     for (int e = lane; e < E; e += Q3_WAVE) z[e] = src[e];
+  } else {
+    for (int e = lane; e < E; e += Q3_WAVE) z[e] = 1.f / (1.f + expf(-src[e])) + correction[e];
   }
   __builtin_amdgcn_wave_barrier();
+  if (mode == 2 && keep < groups) {
+    const int size = E / groups;
+    for (int g = lane; g < groups; g += Q3_WAVE) {          // a group a lane: the sum of its two largest
+      float first = -INFINITY, second = -INFINITY;
+      for (int i = 0; i < size; ++i) {
+        const float c = z[g * size + i];
+        if (c > first) {
+          second = first;
+          first = c;
+        } else if (c > second) {
+          second = c;
+        }
+      }
+      group_score[g] = size > 1 ? first + second : first;
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int k = 0; k < keep; ++k) {                        // the best group left, `keep` times; a kept group's score becomes NaN
+      float best = -INFINITY;
+      int at = 0x7fffffff;
+      for (int g = lane; g < groups; g += Q3_WAVE) {
+        const float p = group_score[g];
+        if (p > best || (at == 0x7fffffff && p == best)) {
+          best = p;
+          at = g;
+        }
+      }
+#pragma unroll
+      for (int off = Q3_WAVE / 2; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, Q3_WAVE);
+        const int oa = __shfl_xor(at, off, Q3_WAVE);
+        if (ob > best || (ob == best && oa < at)) {
+          best = ob;
+          at = oa;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (at < groups) group_score[at] = NAN;
+      __builtin_amdgcn_wave_barrier();
+    }
+    for (int e = lane; e < E; e += Q3_WAVE)
+      if (group_score[e / size] == group_score[e / size]) z[e] = -INFINITY;      // not kept: still a number
+    __builtin_amdgcn_wave_barrier();
+  }
   const float nothing = mode == 0 ? -1.f : -INFINITY;     // below every score that can still be chosen
   float picked_sum = 0.f;
   for (int k = 0; k < top; ++k) {
@@ -67,7 +118,7 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
       }
     }
     if (at >= E) at = 0;          // logits that are no numbers: stay inside the operands
-    const float score = mode == 0 ? best / total : 1.f / (1.f + expf(-best));
+    const float score = mode == 0 ? best / total : 1.f / (1.f + expf(-(mode == 1 ? best : src[at])));
     picked_sum += score;
     __builtin_amdgcn_wave_barrier();
     picked[k] = score;
@@ -553,10 +604,12 @@ __global__ __launch_bounds__(64 * GT_WM * 2) void moe_linear_tiles_kernel(
 
 // out[t, :] = sum_k weights[t, k] * y[slot_of_pair[t * top + k], :] (+ shared[t, :]), float32 sums in
 // the order k = 0, 1, ..., the shared expert last; rounded once. Without `weights` every weight is 1
-// (experts whose inputs carried the weight).
+// (experts whose inputs carried the weight). With `shared_gate` (one float32 logit per token, the
+// tokens' `gate_stride` apart) the shared row is multiplied by sigmoid(shared_gate[t]).
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ slot_of_pair,
                                    const float* __restrict__ weights, const T* __restrict__ shared,
+                                   const float* __restrict__ shared_gate, long gate_stride,
                                    T* __restrict__ out, int width, int top) {
   __shared__ int slots[64];
   __shared__ float share[64];
@@ -573,17 +626,25 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
   for (int k = 0; k < kept; ++k) acc += share[k] * to_float(y[(size_t)slots[k] * width + j]);
   for (int k = kept; k < top; ++k)
     acc += (weights ? weights[(size_t)t * top + k] : 1.f) * to_float(y[(size_t)slot_of_pair[(size_t)t * top + k] * width + j]);
-  if (shared) acc += to_float(shared[(size_t)t * width + j]);
+  if (shared) {
+    const float open = shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * gate_stride])) : 1.f;
+    acc += open * to_float(shared[(size_t)t * width + j]);
+  }
   out[(size_t)t * width + j] = from_float<T>(acc);
 }
 
-extern "C" int q3_moe_pick(const float* logits, int n_tokens, int E, int top, int mode, int* chosen, float* weights,
+extern "C" int q3_moe_pick(const float* logits, long row_stride, int n_tokens, int E, int top, int mode,
+                           const float* correction, int groups, int keep, int* chosen, float* weights,
                            hipStream_t stream) {
-  if (n_tokens <= 0 || E <= 0 || top <= 0 || top > E || E > 4096 || mode < 0 || mode > 1) return Q3_ERR_BAD_ARGUMENT;
+  if (n_tokens <= 0 || E <= 0 || top <= 0 || top > E || E > 4096 || mode < 0 || mode > 2 || row_stride < E)
+    return Q3_ERR_BAD_ARGUMENT;
+  if (mode != 2) groups = keep = 1;
+  if (mode == 2 && (!correction || groups <= 0 || E % groups || keep <= 0 || keep > groups || top > keep * (E / groups)))
+    return Q3_ERR_BAD_ARGUMENT;
   const int waves = 4;
-  const size_t smem = (size_t)waves * (E + top) * sizeof(float);
+  const size_t smem = (size_t)waves * (E + top + groups) * sizeof(float);
   hipLaunchKernelGGL(moe_pick_kernel, dim3((n_tokens + waves - 1) / waves), dim3(waves * Q3_WAVE), smem, stream, logits,
-                     n_tokens, E, top, mode, chosen, weights);
+                     row_stride, n_tokens, E, top, mode, correction, groups, keep, chosen, weights);
   return q3_launch_status();
 }
 
@@ -663,14 +724,16 @@ extern "C" int q3_moe_linear(const void* x, const int* pair_of_slot, int gather,
 }
 
 extern "C" int q3_moe_combine(const void* y, const int* slot_of_pair, const float* weights, const void* shared,
-                              void* out, int n_tokens, int width, int top, int dtype, hipStream_t stream) {
-  if (n_tokens <= 0 || width <= 0 || top <= 0) return Q3_ERR_BAD_ARGUMENT;
+                              const float* shared_gate, long gate_stride, void* out, int n_tokens, int width, int top,
+                              int dtype, hipStream_t stream) {
+  if (n_tokens <= 0 || width <= 0 || top <= 0 || (shared_gate && !shared)) return Q3_ERR_BAD_ARGUMENT;
   int threads = 64;
   while (threads < 256 && threads < width) threads *= 2;
   if ((width + threads - 1) / threads > 65535) return Q3_ERR_UNSUPPORTED;
   Q3_DISPATCH_DTYPE(dtype, TT,
                     hipLaunchKernelGGL(moe_combine_kernel<TT>, dim3(n_tokens, (width + threads - 1) / threads),
                                        dim3(threads), 0, stream, (const TT*)y,
-                                       slot_of_pair, weights, (const TT*)shared, (TT*)out, width, top));
+                                       slot_of_pair, weights, (const TT*)shared, shared_gate, gate_stride, (TT*)out,
+                                       width, top));
   return q3_launch_status();
 }

@@ -214,3 +214,69 @@ extern "C" int q3_rmsnorm_addend(float* x, const void* delta, const void* delta_
   }));
   return Q3_ERR_BAD_ARGUMENT;
 }
+
+// A layer norm with a weight and a bias behind everything the stream still lacks. One block per
+// output row r (source row s):
+//   v = x[s] + delta[s] + extra[s] + vec        (each addend optional: a part's result in the
+//       activation dtype, float32 rows of their own, one float32 vector for every row)
+//   if write_back: x[s] = v
+//   out[r] = (v - mean v) * rsqrt(mean (v - mean v)^2 + eps) * weight + bias
+// The mean is taken first and the deviations are squared afterwards. All float32, the result rounded
+// once; the row lives in shared memory between the passes (`H` floats). Without `weight` only the
+// stream is brought up to date.
+template <typename T>
+__global__ void layernorm_addend_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                        const float* __restrict__ extra, const float* __restrict__ vec,
+                                        const float* __restrict__ weight, const float* __restrict__ bias,
+                                        const int* __restrict__ rows, T* __restrict__ out, int H, int n_src,
+                                        float eps, int write_back) {
+  extern __shared__ float smem[];
+  float* red = smem;
+  float* row = smem + 32;
+  const int r = blockIdx.x;
+  int s = rows ? rows[r] : r;
+  if (s < 0 || s >= n_src) s = 0;
+  float* xs = x + (size_t)s * H;
+  float acc = 0.f;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    float v = xs[j];
+    if (delta) v += to_float(delta[(size_t)s * H + j]);
+    if (extra) v += extra[(size_t)s * H + j];
+    if (vec) v += vec[j];
+    row[j] = v;
+    acc += v;
+    if (write_back) xs[j] = v;
+  }
+  if (!out) return;
+  const float mean = block_sum(acc, red) / (float)H;
+  float sq = 0.f;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    const float d = row[j] - mean;
+    sq += d * d;
+  }
+  const float inv = rsqrtf(block_sum(sq, red) / (float)H + eps);
+  for (int j = threadIdx.x; j < H; j += blockDim.x)
+    out[(size_t)r * H + j] = from_float<T>((row[j] - mean) * inv * weight[j] + (bias ? bias[j] : 0.f));
+}
+
+extern "C" int q3_layernorm_addend(float* x, const void* delta, const float* extra, const float* vec,
+                                   const float* weight, const float* bias, const int* rows, void* out, int n_out,
+                                   int n_src, int H, float eps, int act_dtype, int write_back, hipStream_t stream) {
+  if (n_out <= 0 || n_src <= 0 || H <= 0 || H > 36000) return Q3_ERR_BAD_ARGUMENT;
+  if (write_back && rows) return Q3_ERR_BAD_ARGUMENT;
+  if (out && !weight) return Q3_ERR_BAD_ARGUMENT;
+  int threads = 64;
+  while (threads < 1024 && threads * 4 < H) threads *= 2;
+  const size_t smem = (size_t)(32 + H) * sizeof(float);
+  Q3_DISPATCH_DTYPE(act_dtype, TT, {
+    if (smem > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void*)layernorm_addend_kernel<TT>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL((layernorm_addend_kernel<TT>), dim3(n_out), dim3(threads), smem, stream, x, (const TT*)delta,
+                       extra, vec, weight, bias, rows, (TT*)out, H, n_src, eps, write_back);
+    return q3_launch_status();
+  });
+  return Q3_ERR_BAD_ARGUMENT;
+}

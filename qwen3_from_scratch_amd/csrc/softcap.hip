@@ -5,7 +5,7 @@
 #include "common.h"
 
 // One block per token. The row is [q: H dim | k: G dim | v: G vdim | ...] float32, `bias` covers
-// q, k and v. q and k (bias added) are each divided by the root mean square of the whole
+// q, k and v (null: projections without biases). q and k (bias added) are each divided by the root mean square of the whole
 // projection and multiplied by their weight, then the first 2 * half numbers of every head turn
 // in pairs (2i, 2i + 1) by position * inv_freq[i]. q goes to `q_out`, k and v (bias added) into
 // the token's place in the cache, when one is given.
@@ -22,11 +22,11 @@ __global__ void softcap_prepare_kernel(const float* __restrict__ rows, long row_
   const int nq = H * dim, nk = G * dim, nv = G * vdim;
   float sq = 0.f, sk = 0.f;
   for (int j = threadIdx.x; j < nq; j += blockDim.x) {
-    const float z = row[j] + bias[j];
+    const float z = row[j] + (bias ? bias[j] : 0.f);
     sq += z * z;
   }
   for (int j = threadIdx.x; j < nk; j += blockDim.x) {
-    const float z = row[nq + j] + bias[nq + j];
+    const float z = row[nq + j] + (bias ? bias[nq + j] : 0.f);
     sk += z * z;
   }
   const float rq = rsqrtf(block_sum(sq, scratch) / (float)nq + eps);
@@ -35,10 +35,10 @@ __global__ void softcap_prepare_kernel(const float* __restrict__ rows, long row_
   const float fpos = (float)pos;
   for (int j = threadIdx.x; j < nq; j += blockDim.x) {
     const int e = j % dim;
-    float own = (row[j] + bias[j]) * rq * q_weight[j];
+    float own = (row[j] + (bias ? bias[j] : 0.f)) * rq * q_weight[j];
     if (e < 2 * half) {
       const int p = j ^ 1;
-      const float other = (row[p] + bias[p]) * rq * q_weight[p];
+      const float other = (row[p] + (bias ? bias[p] : 0.f)) * rq * q_weight[p];
       const float angle = fpos * inv_freq[e >> 1];
       const float c = cosf(angle), s = sinf(angle);
       own = (e & 1) ? own * c + other * s : own * c - other * s;
@@ -51,10 +51,10 @@ __global__ void softcap_prepare_kernel(const float* __restrict__ rows, long row_
   const int off = pos % page;
   for (int j = threadIdx.x; j < nk; j += blockDim.x) {
     const int g = j / dim, e = j % dim;
-    float own = (row[nq + j] + bias[nq + j]) * rk * k_weight[j];
+    float own = (row[nq + j] + (bias ? bias[nq + j] : 0.f)) * rk * k_weight[j];
     if (e < 2 * half) {
       const int p = j ^ 1;
-      const float other = (row[nq + p] + bias[nq + p]) * rk * k_weight[p];
+      const float other = (row[nq + p] + (bias ? bias[nq + p] : 0.f)) * rk * k_weight[p];
       const float angle = fpos * inv_freq[e >> 1];
       const float c = cosf(angle), s = sinf(angle);
       own = (e & 1) ? own * c + other * s : own * c - other * s;
@@ -65,7 +65,7 @@ __global__ void softcap_prepare_kernel(const float* __restrict__ rows, long row_
     const int g = j / vdim, e = j % vdim;
     const size_t at = v_transposed ? (((size_t)pg * G + g) * vdim + e) * page + off
                                    : (((size_t)pg * G + g) * page + off) * vdim + e;
-    v_cache[at] = from_float<TA>(row[nq + nk + j] + bias[nq + nk + j]);
+    v_cache[at] = from_float<TA>(row[nq + nk + j] + (bias ? bias[nq + nk + j] : 0.f));
   }
 }
 

@@ -2,7 +2,7 @@
 
 from .decoder import DecoderModel, build_model, expected_tensors
 from .spec import LayerSpec, ModelSpec, RunStep, Slot, pre_norm_layer
-from . import dufinex, kodisun, qwen3, surasun  # noqa: F401
+from . import dufinex, fidevik, kodisun, qwen3, surasun  # noqa: F401
 
 __all__ = ["DecoderModel", "build_model", "expected_tensors", "LayerSpec", "ModelSpec", "RunStep", "Slot",
            "pre_norm_layer"]

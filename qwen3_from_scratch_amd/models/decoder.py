@@ -135,6 +135,8 @@ class DecoderModel:
         what `cache` holds. `cache.view(plane, writes)` gives a mixer its view."""
         x = self.embedding.forward(batch.token_ids)
         x = self.position.on_embeddings(x, batch)
+        # a model whose passes begin with the embedding's output once more keeps a copy: the stream moves on in place
+        start = x.clone() if getattr(self.pass_vectors, "wants_start", False) else None
         pending = None
         order = self.spec.order
         for i, step in enumerate(order):
@@ -144,7 +146,8 @@ class DecoderModel:
             if entry is not None and order[i + 1].enters is not None:
                 entry = None                      # a pass's vector still has to join the stream in between
             if step.enters is not None:
-                pending = self.pass_vectors.join(pending, step.enters)
+                pending = (self.pass_vectors.join(pending, step.enters) if start is None
+                           else self.pass_vectors.join(pending, step.enters, start=start))
             x, pending = self.layers[step.layer].block.forward(x, pending, batch, view,
                                                                next_norm=entry() if entry else None)
             if self.observer is not None:

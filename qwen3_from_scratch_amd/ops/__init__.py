@@ -31,6 +31,9 @@ __all__ = [
     "decode_attention",
     "decode_attention_takes",
     "swiglu",
+    "gated_act",
+    "layernorm_addend",
+    "moe_glu_experts",
     "glu_clamped",
     "gelu",
     "latent_prepare",
@@ -266,9 +269,15 @@ def embed_rows(ids, table, out=None, scale=1.0):
     return out
 
 
-def swiglu(gate_up, out=None):
-    """out[:, j] = silu(gate_up[:, 2j]) * gate_up[:, 2j + 1]: gate and up interleaved, (T, 2I) -> (T, I)."""
+GATE_KINDS = {"silu": 0, "gelu_tanh": 1, "gelu_erf": 2}
+
+
+def gated_act(gate_up, kind="silu", out=None):
+    """out[:, j] = act(gate_up[:, 2j]) * gate_up[:, 2j + 1]: gate and up interleaved, (T, 2I) -> (T, I).
+    `kind`: "silu" for g / (1 + exp(-g)), "gelu_tanh" for 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))),
+    "gelu_erf" for 0.5 g (1 + erf(g / sqrt 2)); float32 arithmetic, rounded once."""
     _dev(gate_up, out)
+    _need(kind in GATE_KINDS, "kind is one of %s" % ", ".join(sorted(GATE_KINDS)))
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0 and gate_up.dtype in _DT,
           "gate_up must be (T, 2I) bfloat16 or float32")
     T, I = gate_up.shape[0], gate_up.shape[1] // 2
@@ -276,9 +285,14 @@ def swiglu(gate_up, out=None):
         out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
     _need(out.shape == (T, I) and out.dtype == gate_up.dtype, "out must be (T, I) of the input's dtype")
     if T:
-        _check(library("elementwise").q3_swiglu(
-            _ptr(gate_up), _ptr(out), T, I, _DT[gate_up.dtype], _stream()), "swiglu")
+        _check(library("elementwise").q3_gated_act(
+            _ptr(gate_up), _ptr(out), T, I, GATE_KINDS[kind], _DT[gate_up.dtype], _stream()), "gated_act")
     return out
+
+
+def swiglu(gate_up, out=None):
+    """out[:, j] = silu(gate_up[:, 2j]) * gate_up[:, 2j + 1]: gate and up interleaved, (T, 2I) -> (T, I)."""
+    return gated_act(gate_up, "silu", out=out)
 
 
 def glu_clamped(gate_up, limit, slope, bias=None, scale=None, scale_index=None, out_dtype=None):
@@ -390,6 +404,41 @@ def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, del
     return out
 
 
+def layernorm_addend(x, weight, bias, eps, out_dtype, delta=None, extra=None, vec=None, rows=None, write_back=True):
+    """A layer norm with a weight and a bias of the float32 stream behind everything the stream still
+    lacks, in float32 and in one kernel. For each output row r (source row s = rows[r], or r):
+
+    v = x[s] + delta[s] + extra[s] + vec, every addend optional: `delta` (T, H) in the activation dtype (a
+    part's result), `extra` float32 (T, H) (rows that join as they are), `vec` float32 (H,) (one vector for
+    every row); x[s] = v if `write_back` and `rows` is None; out[r] = (v - mean(v)) * rsqrt(mean((v -
+    mean(v))^2) + eps) * weight + bias, rounded once to `out_dtype`. `weight` and `bias` are float32 (H,)
+    (`bias` None: none). With `weight` None only the stream is brought up to date and None is returned."""
+    _dev(x, weight, bias, delta, extra, vec, rows)
+    _need(x.dim() == 2 and x.dtype == torch.float32, "x must be float32 (T, H)")
+    T, H = x.shape
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    for w, what in ((weight, "weight"), (bias, "bias"), (vec, "vec")):
+        if w is not None:
+            _f32(w, (H,), what)
+    _need(weight is not None or bias is None, "a bias comes with a weight")
+    if delta is not None:
+        _need(delta.shape == (T, H) and delta.dtype == out_dtype, "delta must be (T, H) of the activation dtype")
+    if extra is not None:
+        _f32(extra, (T, H), "extra")
+    n_out = T
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1, "rows must be int32 (R,)")
+        n_out = rows.shape[0]
+    _need(weight is not None or rows is None, "without a weight there is no output")
+    out = torch.empty((n_out, H), dtype=out_dtype, device=x.device) if weight is not None else None
+    write = 1 if (write_back and rows is None and (delta is not None or extra is not None or vec is not None)) else 0
+    if n_out and (out is not None or write):
+        _check(library("norm").q3_layernorm_addend(
+            _ptr(x), _ptr(delta), _ptr(extra), _ptr(vec), _ptr(weight), _ptr(bias), _ptr(rows), _ptr(out), n_out, T, H,
+            ctypes.c_float(eps), _DT[out_dtype], write, _stream()), "layernorm_addend")
+    return out
+
+
 def gelu(x, kind="erf", out=None):
     """gelu(x) elementwise in float32, rounded once. `kind`: "erf" for 0.5 z (1 + erf(z / sqrt 2)),
     "tanh" for 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))."""
@@ -411,21 +460,26 @@ def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv
                    block_table=None, cache=None):
     """The narrow vectors of latent attention from their joint down-projection, in float32:
 
-    down (T, q_rank + kv_rank + rot_dim) holds [query latent | key/value latent | key part to be
-    rotated]. Returns the normalised query latent (T, q_rank) (`q_weight`, `eps`), and writes
+    down (T, n), n >= q_rank + kv_rank + rot_dim, rows possibly apart, holds [query latent | key/value
+    latent | key part to be rotated | ...]; rot_dim may be 0 (keys without a rotated part; `inv_freq`
+    None). Returns the normalised query latent (T, q_rank) (`q_weight`, `eps`), and writes
     [normalised key/value latent (`kv_weight`) | rotated key part] as the token's row of `cache`
     (pages, page, kv_rank + rot_dim) at page block_table[seq_index[t], position // page]; entries
     below zero are skipped, nothing is written without a cache. The rotation turns the pairs
     (2i, 2i + 1), i < len(inv_freq), by float32(position) * inv_freq[i], with cos and sin
     multiplied by `rot_factor`; what lies beyond the pairs passes."""
-    _dev(down, q_weight, kv_weight, inv_freq, positions, seq_index, block_table, cache)
+    _dev(q_weight, kv_weight, inv_freq, positions, seq_index, block_table, cache)
     R = q_rank + kv_rank + rot_dim
-    _need(down.dim() == 2 and down.shape[1] == R and down.dtype in _DT, "down must be (T, q_rank + kv_rank + rot_dim)")
+    _need(down.is_cuda and down.dim() == 2 and down.shape[1] >= R and down.dtype in _DT and down.stride(1) == 1,
+          "down must be (T, q_rank + kv_rank + rot_dim or more) with its columns side by side")
     T = down.shape[0]
     _need(q_weight.shape == (q_rank,) and kv_weight.shape == (kv_rank,) and q_weight.dtype in _DT
           and kv_weight.dtype == q_weight.dtype, "norm weights (q_rank,) and (kv_rank,) of one dtype")
-    _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 2 * inv_freq.shape[0] <= rot_dim,
-          "inv_freq float32, at most rot_dim / 2 pairs")
+    pairs = 0
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 2 * inv_freq.shape[0] <= rot_dim,
+              "inv_freq float32, at most rot_dim / 2 pairs")
+        pairs = inv_freq.shape[0]
     for t in (positions, seq_index):
         _need(t.dtype == torch.int32 and t.shape == (T,), "positions and seq_index must be int32 (T,)")
     page = pages = stride = rows = 0
@@ -439,8 +493,8 @@ def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv
     cq = torch.empty((T, q_rank), dtype=down.dtype, device=down.device)
     if T:
         _check(library("latent").q3_latent_prepare(
-            _ptr(down), T, q_rank, kv_rank, rot_dim, _ptr(q_weight), _ptr(kv_weight), _DT[q_weight.dtype],
-            ctypes.c_float(eps), _ptr(inv_freq), inv_freq.shape[0], ctypes.c_float(rot_factor), _ptr(positions),
+            _ptr(down), ctypes.c_long(down.stride(0)), T, q_rank, kv_rank, rot_dim, _ptr(q_weight), _ptr(kv_weight),
+            _DT[q_weight.dtype], ctypes.c_float(eps), _ptr(inv_freq), pairs, ctypes.c_float(rot_factor), _ptr(positions),
             _ptr(seq_index), _ptr(block_table), stride, rows, _ptr(cache), page, pages, _ptr(cq), _DT[down.dtype],
             _stream()), "latent_prepare")
     return cq
@@ -488,7 +542,7 @@ def rotate_heads(x, out, inv_freq, rot_factor, positions):
 
 
 def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0,
-                     general=False, max_kv_len=0):
+                     general=False, max_kv_len=0, sink=None, gate=None):
     """Causal softmax attention of every head's query rows over one shared sequence of cached rows.
 
     q (T, H, Dk) contiguous; cache (pages, page, Dk): the row of sequence b's position j lies in
@@ -499,8 +553,11 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
     (up to 576) and value_dim in steps of 16 (up to 512) runs on the matrix cores; everything
     else, and everything with `general=True`, takes the kernel of float32 multiply-adds.
     `max_q_len` bounds the sequences' rows and `max_kv_len` (0: unknown) their keys: a step of few
-    rows over many keys shares the keys out over several blocks per row tile."""
-    _dev(q, cache, block_table, cu_seqlens_q, kv_lens)
+    rows over many keys shares the keys out over several blocks per row tile. `sink` float32 (H,):
+    head h's softmax has exp(sink[h]) as one more term of its denominator, which has no key and no value
+    and is not scaled. `gate` (T, H) of q's dtype, rows possibly apart: head h's result is multiplied by
+    sigmoid(gate[t, h])."""
+    _dev(q, cache, block_table, cu_seqlens_q, kv_lens, sink)
     _need(q.dim() == 3 and q.dtype in _DT and cache.dim() == 3 and cache.dtype == q.dtype
           and cache.shape[2] == q.shape[2], "q (T, H, Dk) and cache (pages, page, Dk) of one dtype")
     T, H, Dk = q.shape
@@ -510,6 +567,12 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
           "cu_seqlens_q int32 (B + 1,), kv_lens int32 (B,)")
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.shape[0] >= B,
           "block_table must be int32 (B, W)")
+    gate_stride = 0
+    if sink is not None:
+        _f32(sink, (H,), "sink")
+    if gate is not None:
+        gate_stride = _rows_view(gate, "gate")
+        _need(gate.shape == (T, H) and gate.dtype == q.dtype, "gate must be (T, H) of q's dtype")
     out = torch.empty((T, H, value_dim), dtype=q.dtype, device=q.device)
     if T and B:
         lib = library("latent")
@@ -521,7 +584,8 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
         _check(lib.q3_latent_attention(
             _ptr(q), _ptr(out), _ptr(cache), cache.shape[0], _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens_q), _ptr(kv_lens), B, T, H, Dk, value_dim, cache.shape[1], ctypes.c_float(scale), int(window),
-            int(max_q_len), _DT[q.dtype], 1 if general else 0, splits, _ptr(partial), _stream()), "latent_attention")
+            int(max_q_len), _DT[q.dtype], 1 if general else 0, splits, _ptr(partial), _ptr(sink), _ptr(gate),
+            ctypes.c_long(gate_stride), _stream()), "latent_attention")
     return out
 
 
@@ -536,30 +600,51 @@ def _latent_splits(T, B, H, max_q_len, max_kv_len, window):
     return max(1, min(512 // tiles, keys // 128, 32))
 
 
-MOE_SCORING = {"softmax": 0, "sigmoid": 1}
+MOE_SCORING = {"softmax": 0, "sigmoid": 1, "sigmoid_groups": 2}
 
 
-def moe_route(h, router, top, tiled=None, scoring="softmax"):
+def moe_route(h, router, top, tiled=None, scoring="softmax", correction=None, groups=1, keep=1, experts=None):
     """Per token the `top` experts with the largest scores and their weights: h (T, width),
     router (E, width) of h's dtype (`tiled`: its tile-ordered copy, if the caller keeps one). The
     logits are a product with float32 sums and a float32 result; scores, the choice and the weights
     are float32. Returns chosen int32 (T, top), in the order of falling score (the lowest index
     among equals), and weights float32 (T, top) = score / (sum of the chosen scores + 1e-20) for
     `scoring` "softmax" (scores = softmax over all experts); with "sigmoid" every expert's score is
-    sigmoid(z) for itself and the weights are the chosen scores as they are."""
-    _dev(h, router)
+    sigmoid(z) for itself and the weights are the chosen scores as they are. With "sigmoid_groups" the
+    choice goes by sigmoid(z) + correction (`correction` float32 (E,)) and only among the experts of `keep`
+    of the `groups` equal groups of neighbouring experts, those groups whose two largest such scores sum
+    highest; the weights are sigmoid(z) of the chosen, without the correction.
+
+    `experts`: the router's first `experts` rows are the experts'; what further rows it has are other
+    numbers per token that ride on the same product (a gate, say), and their float32 results come back
+    as a third value, (T, rows - experts) with rows apart."""
+    _dev(h, router, correction)
     _need(scoring in MOE_SCORING, "scoring is softmax or sigmoid")
     _need(h.dim() == 2 and router.dim() == 2 and h.shape[1] == router.shape[1] and h.dtype in _DT
           and router.dtype == h.dtype, "h (T, width) and router (E, width) of one dtype")
-    T, E = h.shape[0], router.shape[0]
-    _need(1 <= top <= E, "top must lie in 1..E")
+    T, rows = h.shape[0], router.shape[0]
+    E = rows if experts is None else int(experts)
+    _need(1 <= E <= rows and 1 <= top <= E, "experts must lie in 1..rows of the router, top in 1..experts")
+    if scoring == "sigmoid_groups":
+        _need(correction is not None, "the grouped choice needs a correction")
+        _f32(correction, (E,), "correction")
+        _need(groups >= 1 and E % groups == 0 and 1 <= keep <= groups and top <= keep * (E // groups),
+              "groups divide the experts, keep lies in 1..groups, and the kept groups hold at least top experts")
+    else:
+        _need(correction is None and groups == 1 and keep == 1, "a correction and groups belong to sigmoid_groups")
     chosen = torch.empty((T, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    logits = None
     if T:
         logits = linear(h, router, out_dtype=torch.float32, tiled=tiled)
-        _check(library("moe").q3_moe_pick(_ptr(logits), T, E, top, MOE_SCORING[scoring], _ptr(chosen), _ptr(weights),
+        _check(library("moe").q3_moe_pick(_ptr(logits), ctypes.c_long(rows), T, E, top, MOE_SCORING[scoring],
+                                          _ptr(correction), int(groups), int(keep), _ptr(chosen), _ptr(weights),
                                           _stream()), "moe_route")
-    return chosen, weights
+    if experts is None:
+        return chosen, weights
+    if logits is None:
+        logits = torch.empty((0, rows), dtype=torch.float32, device=h.device)
+    return chosen, weights, logits[:, E:]
 
 
 def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
@@ -604,8 +689,8 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
                                  GELU_KINDS[activation], _DT[h.dtype], stream), "moe_linear")
         _check(lib.q3_moe_linear(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff, -1,
                                  _DT[h.dtype], stream), "moe_linear")
-    _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), _ptr(weights), _ptr(shared), _ptr(out), T, width, top,
-                              _DT[h.dtype], stream), "moe_combine")
+    _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), _ptr(weights), _ptr(shared), None, ctypes.c_long(0), _ptr(out),
+                              T, width, top, _DT[h.dtype], stream), "moe_combine")
     return out
 
 
@@ -663,8 +748,61 @@ def moe_gated_experts(h, chosen, weights, gate_up, down, limit, slope):
     else:
         _check(lib.q3_moe_linear(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff, -1,
                                  _DT[h.dtype], stream), "moe_linear")
-    _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), None, None, _ptr(out), T, width, top, _DT[h.dtype], stream),
-           "moe_combine")
+    _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), None, None, None, ctypes.c_long(0), _ptr(out), T, width, top,
+                              _DT[h.dtype], stream), "moe_combine")
+    return out
+
+
+def moe_glu_experts(h, chosen, weights, gate_up, down, activation="silu", shared=None, shared_gate=None):
+    """sum_k weights[t, k] * down[e] (act(gate[e] h[t]) * (up[e] h[t])), e = chosen[t, k]: experts that are
+    gated units without biases, weighted on their results. h (T, width), gate_up (E, 2 ff, width) with rows
+    2j the gate's and 2j + 1 the other branch's, down (E, width, ff), `activation` one of `GATE_KINDS`;
+    `shared` (T, width) is added last, multiplied by sigmoid(shared_gate[t]) when `shared_gate` (float32
+    (T,) or (T, 1), rows possibly apart: a logit per token) is given. Returns (T, width). The pairs are
+    sorted by expert on the GPU as in `moe_experts`; a token's sum is formed in float32 in the order of
+    its choices."""
+    _dev(h, chosen, weights, gate_up, down, shared)
+    T, width = h.shape
+    E, ff = down.shape[0], down.shape[2]
+    top = chosen.shape[1]
+    _need(h.dtype in _DT and gate_up.dtype == h.dtype and down.dtype == h.dtype and gate_up.shape == (E, 2 * ff, width)
+          and down.shape == (E, width, ff), "gate_up (E, 2 ff, width) and down (E, width, ff) of h's dtype")
+    _need(chosen.shape == (T, top) and chosen.dtype == torch.int32 and weights.shape == (T, top)
+          and weights.dtype == torch.float32 and weights.is_contiguous(), "chosen int32 (T, top), weights float32 (T, top)")
+    _need(shared is None or (shared.shape == (T, width) and shared.dtype == h.dtype), "shared (T, width)")
+    _need(activation in GATE_KINDS, "activation is one of %s" % ", ".join(sorted(GATE_KINDS)))
+    gate_stride = 0
+    if shared_gate is not None:
+        _need(shared is not None and shared_gate.is_cuda and shared_gate.dtype == torch.float32
+              and shared_gate.numel() == T and shared_gate.shape[0] == T, "shared_gate float32, one logit per token")
+        gate_stride = shared_gate.stride(0)
+    out = torch.empty((T, width), dtype=h.dtype, device=h.device)
+    if not T:
+        return out
+    lib = library("moe")
+    P = T * top
+    cores = h.dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
+    many = 3 if width % 64 == 0 and ff % 64 == 0 else 2
+    tile_rows = lib.q3_moe_tile_rows((many if P >= 96 * E else 1) if cores else 0)
+    tiles, pair_of_slot, slot_of_pair = _moe_book(lib, chosen, E, tile_rows)
+    both = torch.empty((P, 2 * ff), dtype=h.dtype, device=h.device)
+    y = torch.empty((P, width), dtype=h.dtype, device=h.device)
+    stream = _stream()
+    if cores:
+        _check(lib.q3_moe_linear_mma(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(both), *tiles, 2 * ff, width,
+                                     -1, tile_rows, stream), "moe_linear")
+    else:
+        _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(both), *tiles, 2 * ff, width, -1,
+                                 _DT[h.dtype], stream), "moe_linear")
+    hidden = gated_act(both, activation)
+    if cores:
+        _check(lib.q3_moe_linear_mma(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff,
+                                     -1, tile_rows, stream), "moe_linear")
+    else:
+        _check(lib.q3_moe_linear(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff, -1,
+                                 _DT[h.dtype], stream), "moe_linear")
+    _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), _ptr(weights), _ptr(shared), _ptr(shared_gate),
+                              ctypes.c_long(gate_stride), _ptr(out), T, width, top, _DT[h.dtype], stream), "moe_combine")
     return out
 
 
@@ -930,7 +1068,7 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
     """Queries, keys and values of a step from the float32 rows of their joint product.
 
     rows float32 (T, n), n >= heads dim + kv_heads dim + kv_heads vdim, laid out [q | k | v | ...];
-    bias float32 over q, k and v is added; q and k are each divided by the root mean square of the
+    bias float32 over q, k and v is added (None: projections without biases); q and k are each divided by the root mean square of the
     whole projection and multiplied by `q_weight` (heads dim) and `k_weight` (kv_heads dim); the
     first 2 len(inv_freq) numbers of every head turn in pairs (2i, 2i + 1) by position * inv_freq[i].
     Returns q (T, heads, dim) of `out_dtype`; with a cache, keys (pages, kv_heads, page, dim) and
@@ -941,7 +1079,8 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
     T = rows.shape[0]
     nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
     _need(rows.shape[1] >= nq + nk + nv and heads % kv_heads == 0, "rows hold q, k and v; kv_heads divides heads")
-    _f32(bias, (nq + nk + nv,), "bias")
+    if bias is not None:
+        _f32(bias, (nq + nk + nv,), "bias")
     _f32(q_weight, (nq,), "q_weight")
     _f32(k_weight, (nk,), "k_weight")
     half = 0

@@ -159,8 +159,9 @@ class StreamAddend:
     """What the residual stream still lacks when a norm reads it next: `values` (T, width) in the
     activation dtype, a part's result, which is first normalised by its root mean square with
     `weight` and `eps` if `weight` is given (a block that also normalises what its parts return);
-    and `bias` (width,) float32, one vector for every row (what a model adds to the stream
-    between two layers). Either may be None. `values_bias` (width,) float32 belongs to the part's
+    `bias` (width,) float32, one vector for every row (what a model adds to the stream
+    between two layers); and `extra` (T, width) float32, rows that join as they are (what a model
+    adds row by row: the embedding's output once more, say). Any may be None. `values_bias` (width,) float32 belongs to the part's
     result itself (the bias of its last product, see `BiasedRows`) and joins `values` before their
     norm. A norm that takes it as `delta` does the whole sum in float32 in its own kernel, so the
     addend is never rounded on its way into the stream."""
@@ -170,6 +171,7 @@ class StreamAddend:
     eps: float = 0.0
     bias: torch.Tensor = None
     values_bias: torch.Tensor = None
+    extra: torch.Tensor = None
 
 
 @dataclass

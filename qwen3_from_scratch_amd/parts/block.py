@@ -13,7 +13,7 @@ def _says(part, what):
 @register_part("block", "pre_norm")
 class PreNormBlock(Part):
     """x = x + mixer(norm_1(x)); x = x + feed_forward(norm_2(x))
-    (src/qwen3_from_scratch/models/transformer_block.py:38-46).
+    (src/qwen3_from_scratch/models/transformer_block.py:38-46); a layer may lack the second half.
 
     The residual stream x is float32. The second addition is handed to whoever
     normalises next, so that each addition is fused with the norm that follows
@@ -29,9 +29,12 @@ class PreNormBlock(Part):
         super().__init__(prefix, precision, device)
         self.mixer = self.feed_forward = self.mixer_norm = self.feed_forward_norm = None
 
-    def attach(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+    def attach(self, mixer, mixer_norm, feed_forward=None, feed_forward_norm=None):
         """The layer's parts, under the names its LayerSpec gave them: a block's `attach` names
-        the parts it arranges as its keywords, and a layer that brings others does not build."""
+        the parts it arranges as its keywords, and a layer that brings others does not build. A
+        layer without a feed-forward attaches the mixer and its norm only."""
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("a feed-forward comes with its norm, or not at all")
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.mixer_norm = mixer_norm
@@ -49,10 +52,12 @@ class PreNormBlock(Part):
         reader takes UnscaledRows. Returns the stream and the next `pending`."""
         h = pending if isinstance(pending, UnscaledRows) else self.mixer_norm.forward(x, delta=pending)
         sink = None
-        if (_says(self.mixer, "feeds_sink") and _says(self.feed_forward, "takes_unscaled")
+        if (self.feed_forward is not None and _says(self.mixer, "feeds_sink") and _says(self.feed_forward, "takes_unscaled")
                 and hasattr(self.feed_forward_norm, "sink_for")):
             sink = self.feed_forward_norm.sink_for(x)
         d = self.mixer.forward(h, batch, cache, sink=sink) if sink is not None else self.mixer.forward(h, batch, cache)
+        if self.feed_forward is None:
+            return x, d
         h = d if isinstance(d, UnscaledRows) else self.feed_forward_norm.forward(x, delta=d)
         sink = next_norm.sink_for(x) if next_norm is not None and _says(self.feed_forward, "feeds_sink") else None
         if sink is not None:

@@ -43,14 +43,22 @@ class PassVectors(Part):
     """One vector per pass of a run of layers that a model goes through several times with the
     same weights: a table (passes, hidden_size), of which row t is added to every row of the
     residual stream before pass t begins. The addition itself is left to the norm that reads the
-    stream next (`join` hands it on as part of a `StreamAddend`), in float32."""
+    stream next (`join` hands it on as part of a `StreamAddend`), in float32. With `restart` every
+    pass but the first also begins with the embedding's output added to the stream once more, rows
+    that the model keeps for this (`wants_start`) and that travel the same way."""
 
     graph_safe = True
 
-    def __init__(self, prefix, precision, device, passes, hidden_size, leaf="weight"):
+    def __init__(self, prefix, precision, device, passes, hidden_size, leaf="weight", restart=False):
         super().__init__(prefix, precision, device)
         self.passes, self.hidden_size, self.leaf = passes, hidden_size, leaf
+        self.restart = bool(restart)
         self.table = None
+
+    @property
+    def wants_start(self):
+        """Whether `join` needs the stream as the embedding left it (a copy: the stream itself moves on)."""
+        return self.restart and self.passes > 1
 
     def tensors(self):
         return {self._name(self.leaf): (self.passes, self.hidden_size)}
@@ -58,17 +66,23 @@ class PassVectors(Part):
     def load(self, fetch):
         self.table = fetch(self._name(self.leaf), torch.float32).contiguous()
 
-    def join(self, pending, number):
+    def join(self, pending, number, start=None):
         """`pending` (what the stream still lacks: None, a tensor or a StreamAddend) with pass
-        `number`'s vector added to it."""
+        `number`'s vector added to it and, with `restart`, for every pass but the first also `start`,
+        the float32 rows the embedding gave."""
         row = self.table[number]
+        extra = None
+        if self.restart and number > 0:
+            if start is None:
+                raise ValueError("pass %d begins with the embedding's output once more, which was not kept" % number)
+            extra = start
         if pending is None:
-            return StreamAddend(bias=row)
+            return StreamAddend(bias=row, extra=extra)
         if isinstance(pending, UnscaledRows):
             raise ValueError("a pass cannot begin behind rows whose addition is already done")
         if isinstance(pending, StreamAddend):
-            if pending.bias is not None:
+            if pending.bias is not None or pending.extra is not None:
                 raise ValueError("two vectors wait for the same place of the stream")
             return StreamAddend(values=pending.values, weight=pending.weight, eps=pending.eps, bias=row,
-                                values_bias=pending.values_bias)
-        return StreamAddend(values=pending, bias=row)
+                                values_bias=pending.values_bias, extra=extra)
+        return StreamAddend(values=pending, bias=row, extra=extra)

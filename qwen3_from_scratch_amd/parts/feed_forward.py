@@ -15,14 +15,19 @@ class SwiGLU(Part):
     one matrix with their rows interleaved (row 2i gate's, row 2i + 1 up's), so
     that one product feeds the activation, which for few rows is the product
     kernel's epilogue (the reference's fused variant concatenates them,
-    feedback.py:52-54)."""
+    feedback.py:52-54). `activation`: what the gate passes, "silu" or one of the other kinds of
+    `ops.GATE_KINDS` (the tanh form of gelu, the exact gelu), which run as the plain product and an
+    activation kernel behind it."""
 
     graph_safe = True
     feeds_sink = True
 
     def __init__(self, prefix, precision, device, hidden_size, intermediate_size,
-                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight"), activation="silu"):
         super().__init__(prefix, precision, device)
+        if activation not in ops.GATE_KINDS:
+            raise ValueError("activation is one of %s" % ", ".join(sorted(ops.GATE_KINDS)))
+        self.activation = activation
         self.names = tuple(names)         # the tensors' names below the prefix: gate, up, down
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
@@ -46,10 +51,13 @@ class SwiGLU(Part):
 
     @property
     def takes_unscaled(self):
-        return self.gate_up is not None and self.gate_up.fuses
+        return self.activation == "silu" and self.gate_up is not None and self.gate_up.fuses
 
     def forward(self, x, batch=None, sink=None):
-        h = self.gate_up.forward_swiglu(x)
+        if self.activation == "silu":
+            h = self.gate_up.forward_swiglu(x)
+        else:
+            h = ops.gated_act(self.gate_up.forward(x), self.activation)
         return self.down.forward(h) if sink is None else self.down.forward_into(h, sink)
 
 

@@ -12,12 +12,14 @@ from .linear import LinearWeight
 class LinearHead(Part):
     """logits = h @ W^T, no bias (src/qwen3_from_scratch/models/qwen3.py:63-65,83-84).
     `weight_name` is the full checkpoint name of W: the embedding's name ties
-    the head to it (qwen3.py:69-70) and both then share one tensor."""
+    the head to it (qwen3.py:69-70) and both then share one tensor. `scale`: a constant the
+    float32 logits are multiplied by (1: none)."""
 
     graph_safe = True
 
-    def __init__(self, prefix, precision, device, hidden_size, vocab_size, weight_name):
+    def __init__(self, prefix, precision, device, hidden_size, vocab_size, weight_name, scale=1.0):
         super().__init__(prefix, precision, device)
+        self.scale = float(scale)
         self.hidden_size = hidden_size
         self.vocab_size = vocab_size
         self.weight_name = weight_name
@@ -30,4 +32,5 @@ class LinearHead(Part):
         self.weight = LinearWeight(fetch(self.weight_name, self.precision.act), self.precision)
 
     def forward(self, h):
-        return self.weight.forward(h, out_dtype=torch.float32)
+        logits = self.weight.forward(h, out_dtype=torch.float32)
+        return logits if self.scale == 1.0 else logits.mul_(self.scale)

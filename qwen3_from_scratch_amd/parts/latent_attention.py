@@ -25,6 +25,12 @@ class LatentAttention(Part):
     numbers with the softmax weights, and the head's value matrix multiplies that sum. The two
     down-projections are one matrix. Norms, rotation, scores and sums are float32.
 
+    With `rot_dim` 0 keys have no rotated part, positions do not enter the scores and the layer needs
+    no position part. With `sink` the softmax's denominator of head a also holds exp(sink_a), a
+    learned number per head (`sink`, (heads,)) that has no key and no value and is not scaled. With
+    `gated` head a's result is multiplied by sigmoid(W_g h)_a (`g`, (heads, hidden)), a gate that reads
+    the mixer's own input and rides on the down-projections' product.
+
     Tensors (under the part's prefix): dq (q_rank, hidden), dq.norm (q_rank), uq (heads (dim +
     rot_dim), q_rank), dkv (kv_rank + rot_dim, hidden), dkv.norm (kv_rank), uk (heads dim,
     kv_rank), uv (heads vdim, kv_rank), o (hidden, heads vdim). The rotation's frequencies come
@@ -34,15 +40,19 @@ class LatentAttention(Part):
     graph_safe = True
 
     def __init__(self, prefix, precision, device, hidden_size, heads, dim, rot_dim, vdim, q_rank, kv_rank, scale,
-                 eps, window=0):
+                 eps, window=0, sink=False, gated=False):
         super().__init__(prefix, precision, device)
         self.hidden_size, self.heads, self.dim, self.rot_dim, self.vdim = hidden_size, heads, dim, rot_dim, vdim
         self.q_rank, self.kv_rank = q_rank, kv_rank
         self.scale, self.eps, self.window = float(scale), float(eps), int(window)
+        self.has_sink, self.gated = bool(sink), bool(gated)
+        self.sink = None
         self.position = None
         self.down = self.uq = self.uk = self.uv = self.out = self.q_norm = self.kv_norm = None
 
     def attach_position(self, position):
+        if not self.rot_dim:
+            return
         if not hasattr(position, "frequencies"):
             raise ValueError("latent attention rotates by frequencies; the position part %s has none"
                              % type(position).__name__)
@@ -54,7 +64,7 @@ class LatentAttention(Part):
 
     def tensors(self):
         H, W = self.heads, self.hidden_size
-        return {
+        names = {
             self._name("dq"): (self.q_rank, W),
             self._name("dq.norm"): TensorShape((self.q_rank,), "scale"),
             self._name("uq"): (H * (self.dim + self.rot_dim), self.q_rank),
@@ -64,10 +74,16 @@ class LatentAttention(Part):
             self._name("uv"): (H * self.vdim, self.kv_rank),
             self._name("o"): (W, H * self.vdim),
         }
+        if self.has_sink:
+            names[self._name("sink")] = TensorShape((H,), "bias")
+        if self.gated:
+            names[self._name("g")] = (H, W)
+        return names
 
     def load(self, fetch):
         act, H = self.precision.act, self.heads
-        down = torch.cat((fetch(self._name("dq"), act, keep=False), fetch(self._name("dkv"), act, keep=False)), dim=0)
+        down = torch.cat([fetch(self._name(n), act, keep=False) for n in (("dq", "dkv", "g") if self.gated else ("dq", "dkv"))],
+                         dim=0)
         self.down = LinearWeight(down.contiguous(), self.precision)
         self.uq = LinearWeight(fetch(self._name("uq"), act), self.precision)
         # per head (result index, summed index): uk transposed (it is applied to the query), uv as stored
@@ -76,10 +92,12 @@ class LatentAttention(Part):
         self.out = LinearWeight(fetch(self._name("o"), act), self.precision)
         self.q_norm = fetch(self._name("dq.norm"))
         self.kv_norm = fetch(self._name("dkv.norm"))
+        if self.has_sink:
+            self.sink = fetch(self._name("sink"), torch.float32).contiguous()
 
     def forward(self, x, batch, cache):
         H, dn, dr, rank = self.heads, self.dim, self.rot_dim, self.kv_rank
-        inv_freq, factor = self.position.frequencies()
+        inv_freq, factor = self.position.frequencies() if dr else (None, 1.0)
         latent = cache.paged["latent"]
         down = self.down.forward(x)
         cq = ops.latent_prepare(down, self.q_rank, rank, dr, self.q_norm, self.kv_norm, self.eps, inv_freq, factor,
@@ -89,8 +107,11 @@ class LatentAttention(Part):
         q = self.uq.forward(cq).view(-1, H, dn + dr)
         rows = torch.empty((q.shape[0], H, rank + dr), dtype=q.dtype, device=q.device)
         ops.headwise_linear(q[:, :, :dn], self.uk, out=rows[:, :, :rank])
-        ops.rotate_heads(q[:, :, dn:], rows[:, :, rank:], inv_freq, factor, batch.positions)
+        if dr:
+            ops.rotate_heads(q[:, :, dn:], rows[:, :, rank:], inv_freq, factor, batch.positions)
+        at = self.q_rank + rank + dr
         mixed = ops.latent_attention(rows, latent, rank, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
-                                     batch.max_q_len, self.scale, window=self.window, max_kv_len=batch.max_kv_len)
+                                     batch.max_q_len, self.scale, window=self.window, max_kv_len=batch.max_kv_len,
+                                     sink=self.sink, gate=down[:, at:at + H] if self.gated else None)
         o = ops.headwise_linear(mixed, self.uv)
         return self.out.forward(o.view(-1, H * self.vdim))

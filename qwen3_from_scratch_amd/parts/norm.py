@@ -7,6 +7,12 @@ from ..config.registry import register_part
 from .base import BiasedRows, HyperAddend, NormSink, Part, StreamAddend, TensorShape
 
 
+def _no_extra_rows(addend, norm):
+    if addend.extra is not None:
+        raise ValueError("%s takes no rows of their own among what the stream still lacks; the norm "
+                         "'layer_bias' does" % type(norm).__name__)
+
+
 @register_part("norm", "rms")
 class RMSNorm(Part):
     """y = x * rsqrt(mean(x^2) + eps) * weight, eps inside the root, plain weight
@@ -34,6 +40,7 @@ class RMSNorm(Part):
         """Normalised rows in the activation dtype. With `delta`, x += delta
         first (in place, unless `rows` selects a subset: then x is left alone)."""
         if isinstance(delta, StreamAddend):
+            _no_extra_rows(delta, self)
             return ops.rmsnorm_addend(x, self.weight, self.eps, self.precision.act, delta=delta.values,
                                       delta_weight=delta.weight, delta_eps=delta.eps, bias=delta.bias, rows=rows,
                                       write_back=rows is None, delta_bias=delta.values_bias)
@@ -78,6 +85,7 @@ class StreamReader(Part):
     def forward(self, x, delta=None, rows=None):
         if not isinstance(delta, StreamAddend):
             delta = StreamAddend(values=delta)
+        _no_extra_rows(delta, self)
         return ops.rmsnorm_addend(x, None, 0.0, self.precision.act, delta=delta.values, delta_weight=delta.weight,
                                   delta_eps=delta.eps, bias=delta.bias, rows=rows, write_back=rows is None,
                                   delta_bias=delta.values_bias, plain=True)
@@ -119,3 +127,46 @@ class LayerNorm(Part):
             values, mix, write = delta, self._one, self._one[0]
         return ops.hyper_norm(streams, self.weight, self.eps, self.precision.act, read=read, delta=values, mix=mix,
                               write=write, rows=rows, write_back=rows is None)
+
+
+@register_part("norm", "layer_bias")
+class BiasedLayerNorm(Part):
+    """y = (x - mean(x)) * rsqrt(var(x) + eps) * weight + bias, var the mean of the squared deviations
+    (the mean is taken out first), over the float32 residual stream (T, width). Like the other norms it
+    folds what the stream still lacks into its pass: a part's result (a tensor in the activation
+    dtype), or a `StreamAddend` whose result, vector for every row and float32 rows of their own all
+    join in float32 in the one kernel, before the norm; a result that is itself to be normalised
+    first is not taken. The weight is the tensor `leaf` under the prefix ("" for the prefix itself),
+    the bias the same name with `bias_suffix` added; both are used as float32."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device, size, eps, leaf="weight", bias_suffix=".b"):
+        super().__init__(prefix, precision, device)
+        self.size, self.eps, self.leaf, self.bias_suffix = size, float(eps), leaf, bias_suffix
+        self.weight = self.bias = None
+
+    def tensors(self):
+        name = self._name(self.leaf)
+        return {name: TensorShape((self.size,), "scale"), name + self.bias_suffix: TensorShape((self.size,), "bias")}
+
+    def load(self, fetch):
+        name = self._name(self.leaf)
+        self.weight = fetch(name, torch.float32).contiguous()
+        self.bias = fetch(name + self.bias_suffix, torch.float32).contiguous()
+
+    def forward(self, x, delta=None, rows=None):
+        """Normalised rows in the activation dtype. With `delta`, the stream is brought up to date first
+        (in place, unless `rows` selects a subset: then x is left alone)."""
+        values = extra = vec = None
+        if isinstance(delta, StreamAddend):
+            if delta.weight is not None or delta.values_bias is not None:
+                raise ValueError("BiasedLayerNorm adds a result as it is: it neither normalises it first nor "
+                                 "carries a bias of its last product")
+            values, extra, vec = delta.values, delta.extra, delta.bias
+        elif isinstance(delta, BiasedRows):
+            values = delta.finished()
+        elif delta is not None:
+            values = delta
+        return ops.layernorm_addend(x, self.weight, self.bias, self.eps, self.precision.act, delta=values, extra=extra,
+                                    vec=vec, rows=rows, write_back=rows is None)

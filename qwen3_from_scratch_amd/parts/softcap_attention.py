@@ -19,7 +19,8 @@ class SoftcapAttention(Part):
     (2i, 2i + 1), frequency rot_base^(-2i / rot_dims). score = (q . k) scale, then
     softcap * tanh(score / softcap) (softcap 0: as it is); softmax over the keys at positions
     j <= i (the last `window` of them, 0: all); head a's result is multiplied by sigmoid(W_g h)_a
-    before the output product. The four products are one and leave float32 rows, so biases and
+    before the output product. `biases` false: the three projections have no biases (no `.b` tensors);
+    `gated` false: no gate (no `g`). The products are one and leave float32 rows, so biases and
     norms see unrounded numbers; norms, angles, scores and the softmax are float32. Keys (rotated)
     and values are paged, a page of keys (kv_heads, page, dim) and a page of values (kv_heads, vdim,
     page), transposed within the page as the matrix-core attention kernels read them: bfloat16 with
@@ -28,7 +29,7 @@ class SoftcapAttention(Part):
     graph_safe = True
 
     def __init__(self, prefix, precision, device, hidden_size, heads, kv_heads, dim, vdim, scale, eps, softcap=0.0,
-                 rot_dims=0, rot_base=1.0, window=0):
+                 rot_dims=0, rot_base=1.0, window=0, biases=True, gated=True):
         super().__init__(prefix, precision, device)
         if heads % kv_heads:
             raise ValueError("heads (%d) must be a multiple of kv_heads (%d)" % (heads, kv_heads))
@@ -38,6 +39,7 @@ class SoftcapAttention(Part):
         self.hidden_size, self.heads, self.kv_heads, self.dim, self.vdim = hidden_size, heads, kv_heads, dim, vdim
         self.scale, self.eps, self.softcap, self.window = float(scale), float(eps), float(softcap), int(window)
         self.rot_dims, self.rot_base = int(rot_dims), float(rot_base)
+        self.biases, self.gated = bool(biases), bool(gated)
         self.w_in = self.w_out = self.bias = self.q_norm = self.k_norm = self.inv_freq = None
 
     def cache_need(self):
@@ -46,18 +48,24 @@ class SoftcapAttention(Part):
 
     def tensors(self):
         H, G, d, dv, W = self.heads, self.kv_heads, self.dim, self.vdim, self.hidden_size
-        return {self._name("q"): (H * d, W), self._name("q.b"): TensorShape((H * d,), "bias"),
-                self._name("k"): (G * d, W), self._name("k.b"): TensorShape((G * d,), "bias"),
-                self._name("v"): (G * dv, W), self._name("v.b"): TensorShape((G * dv,), "bias"),
-                self._name("q.norm"): TensorShape((H * d,), "scale"), self._name("k.norm"): TensorShape((G * d,), "scale"),
-                self._name("g"): (H, W), self._name("o"): (W, H * dv)}
+        names = {self._name("q"): (H * d, W), self._name("k"): (G * d, W), self._name("v"): (G * dv, W),
+                 self._name("q.norm"): TensorShape((H * d,), "scale"), self._name("k.norm"): TensorShape((G * d,), "scale"),
+                 self._name("o"): (W, H * dv)}
+        if self.biases:
+            names.update({self._name("q.b"): TensorShape((H * d,), "bias"), self._name("k.b"): TensorShape((G * d,), "bias"),
+                          self._name("v.b"): TensorShape((G * dv,), "bias")})
+        if self.gated:
+            names[self._name("g")] = (H, W)
+        return names
 
     def load(self, fetch):
         act = self.precision.act
-        joined = torch.cat([fetch(self._name(n), act, keep=False) for n in ("q", "k", "v", "g")], dim=0)
+        joined = torch.cat([fetch(self._name(n), act, keep=False)
+                            for n in (("q", "k", "v", "g") if self.gated else ("q", "k", "v"))], dim=0)
         self.w_in = LinearWeight(joined.contiguous(), self.precision)
         self.w_out = LinearWeight(fetch(self._name("o"), act), self.precision)
-        self.bias = torch.cat([fetch(self._name(n + ".b"), torch.float32) for n in ("q", "k", "v")]).contiguous()
+        if self.biases:
+            self.bias = torch.cat([fetch(self._name(n + ".b"), torch.float32) for n in ("q", "k", "v")]).contiguous()
         self.q_norm = fetch(self._name("q.norm"), torch.float32)
         self.k_norm = fetch(self._name("k.norm"), torch.float32)
         self.inv_freq = rotation_frequencies(self.rot_dims, self.rot_base, self.device)
@@ -73,7 +81,8 @@ class SoftcapAttention(Part):
                                 values_transposed=True)
         mixed = ops.softcap_attention(q, keys, values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
                                       batch.seq_index, batch.positions, batch.max_q_len, batch.max_kv_len, self.scale,
-                                      self.softcap, window=self.window, gate=rows[:, (H + G) * d + G * dv:],
+                                      self.softcap, window=self.window,
+                                      gate=rows[:, (H + G) * d + G * dv:] if self.gated else None,
                                       values_transposed=True, min_q_len=batch.min_q_len,
                                       max_kv_len_of_many=getattr(batch, "max_kv_len_portions", None))
         return self.w_out.forward(mixed)

@@ -20,14 +20,46 @@ def embed_rows(ids, table, out=None, scale=1.0):
     return res
 
 
-def swiglu(gate_up, out=None):
+GATE_KINDS = {"silu": 0, "gelu_tanh": 1, "gelu_erf": 2}
+
+
+def gated_act(gate_up, kind="silu", out=None):
     g = gate_up[:, 0::2].float()          # gate and up interleaved
     u = gate_up[:, 1::2].float()
-    res = (g / (1.0 + torch.exp(-g)) * u).to(gate_up.dtype)
+    if kind == "silu":
+        a = g / (1.0 + torch.exp(-g))
+    elif kind == "gelu_tanh":
+        a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g ** 3)))
+    else:
+        a = 0.5 * g * (1.0 + torch.erf(g / math.sqrt(2.0)))
+    res = (a * u).to(gate_up.dtype)
     if out is not None:
         out.copy_(res)
         return out
     return res
+
+
+def swiglu(gate_up, out=None):
+    return gated_act(gate_up, "silu", out=out)
+
+
+def layernorm_addend(x, weight, bias, eps, out_dtype, delta=None, extra=None, vec=None, rows=None, write_back=True):
+    src = x if rows is None else x[rows.long()]
+    if delta is not None:
+        src = src + (delta if rows is None else delta[rows.long()]).float()
+    if extra is not None:
+        src = src + (extra if rows is None else extra[rows.long()])
+    if vec is not None:
+        src = src + vec
+    if write_back and rows is None and (delta is not None or extra is not None or vec is not None):
+        x.copy_(src)
+    if weight is None:
+        return None
+    dev = src - src.mean(dim=-1, keepdim=True)
+    res = dev * torch.rsqrt((dev * dev).mean(dim=-1, keepdim=True) + eps) * weight
+    if bias is not None:
+        res = res + bias
+    return res.to(out_dtype)
 
 
 def rmsnorm(x, weight, eps, out_dtype, delta=None, rows=None, write_back=True, out=None):
@@ -244,11 +276,12 @@ def _turn_pairs(t, positions, inv_freq, rot_factor):
 def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv_freq, rot_factor, positions, seq_index,
                    block_table=None, cache=None):
     x = down.float()
-    a, b, tail = x[:, :q_rank], x[:, q_rank:q_rank + kv_rank], x[:, q_rank + kv_rank:]
+    a, b, tail = x[:, :q_rank], x[:, q_rank:q_rank + kv_rank], x[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim]
     cq = a * torch.rsqrt((a * a).mean(dim=-1, keepdim=True) + eps) * q_weight.float()
     if cache is not None:
         c = b * torch.rsqrt((b * b).mean(dim=-1, keepdim=True) + eps) * kv_weight.float()
-        row = torch.cat((c, _turn_pairs(tail, positions, inv_freq, rot_factor)), dim=-1)
+        row = torch.cat((c, _turn_pairs(tail, positions, inv_freq, rot_factor)), dim=-1) if inv_freq is not None \
+            else torch.cat((c, tail), dim=-1)
         page = cache.shape[1]
         pos = positions.long()
         pages = block_table[seq_index.long(), pos // page].long()
@@ -270,7 +303,8 @@ def rotate_heads(x, out, inv_freq, rot_factor, positions):
     return out
 
 
-def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0, general=False, max_kv_len=0):
+def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0, general=False,
+                     max_kv_len=0, sink=None, gate=None):
     T, H, Dk = q.shape
     page = cache.shape[1]
     res = torch.zeros((T, H, value_dim), dtype=torch.float32, device=q.device)
@@ -289,13 +323,34 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
         if window > 0:
             hidden = hidden | (qpos - kpos >= window)
         s = torch.einsum("thd,sd->hts", q[q0:q1].float(), rows) * scale
-        p = torch.softmax(s.masked_fill(hidden[None], float("-inf")), dim=-1)
+        s = s.masked_fill(hidden[None], float("-inf"))
+        if sink is not None:
+            s = torch.cat((s, sink.float()[:, None, None].expand(H, n, 1)), dim=-1)
+        p = torch.softmax(s, dim=-1)[..., :L]
         res[q0:q1] = torch.einsum("hts,sd->thd", p, rows[:, :value_dim])
+    if gate is not None:
+        res = res * torch.sigmoid(gate.float())[:, :, None]
     return res.to(q.dtype)
 
 
-def moe_route(h, router, top, tiled=None, scoring="softmax"):
+def moe_route(h, router, top, tiled=None, scoring="softmax", correction=None, groups=1, keep=1, experts=None):
     z = h.float() @ router.float().T
+    if experts is not None:
+        chosen, weights = moe_route(h, router[:experts], top, scoring=scoring, correction=correction, groups=groups, keep=keep)
+        return chosen, weights, z[:, experts:]
+    if scoring == "sigmoid_groups":
+        T, E = z.shape
+        score = torch.sigmoid(z)
+        choice = score + correction
+        if keep < groups:
+            size = E // groups
+            grouped = choice.view(T, groups, size)
+            of_group = grouped.topk(min(2, size), dim=-1).values.sum(dim=-1)
+            kept = torch.zeros((T, groups), dtype=torch.bool)
+            kept[torch.arange(T)[:, None], of_group.topk(keep, dim=-1).indices] = True
+            choice = grouped.masked_fill(~kept[:, :, None], float("-inf")).reshape(T, E)
+        chosen = choice.topk(top, dim=-1).indices
+        return chosen.to(torch.int32), score.gather(1, chosen)
     if scoring == "sigmoid":
         best, chosen = torch.topk(z, top, dim=-1)
         return chosen.to(torch.int32), torch.sigmoid(best)
@@ -312,6 +367,19 @@ def moe_gated_experts(h, chosen, weights, gate_up, down, limit, slope):
         both = torch.einsum("ti,tfi->tf", h.float(), gate_up[e].float()).to(h.dtype)
         hidden = glu_clamped(both, limit, slope, scale=weights[:, k].contiguous())
         out += torch.einsum("tf,twf->tw", hidden.float(), down[e].float()).to(h.dtype).float()
+    return out.to(h.dtype)
+
+
+def moe_glu_experts(h, chosen, weights, gate_up, down, activation="silu", shared=None, shared_gate=None):
+    T, top = chosen.shape
+    out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
+    for k in range(top):
+        e = chosen[:, k].long()
+        both = torch.einsum("ti,tfi->tf", h.float(), gate_up[e].float()).to(h.dtype)
+        y = torch.einsum("tf,twf->tw", gated_act(both, activation).float(), down[e].float()).to(h.dtype)
+        out += weights[:, k, None] * y.float()
+    if shared is not None:
+        out += shared.float() * (torch.sigmoid(shared_gate.reshape(T, 1)) if shared_gate is not None else 1.0)
     return out.to(h.dtype)
 
 
@@ -470,7 +538,9 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
                     out_dtype, block_table=None, k_cache=None, v_cache=None, values_transposed=False):
     T = rows.shape[0]
     nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
-    z = rows[:, :nq + nk + nv].float() + bias.float()
+    z = rows[:, :nq + nk + nv].float()
+    if bias is not None:
+        z = z + bias.float()
     q, k, v = z[:, :nq], z[:, nq:nq + nk], z[:, nq + nk:]
     q = q * torch.rsqrt((q * q).mean(dim=-1, keepdim=True) + eps) * q_weight.float()
     k = k * torch.rsqrt((k * k).mean(dim=-1, keepdim=True) + eps) * k_weight.float()
@@ -576,7 +646,7 @@ def scaled_sum(a, alpha, b, beta):
     return (alpha * a.float() + beta * b.float()).to(a.dtype)
 
 
-ALL = ("glu_clamped", "moe_gated_experts", "headnorm_prepare", "channel_delta", "embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
+ALL = ("gated_act", "GATE_KINDS", "layernorm_addend", "moe_glu_experts", "glu_clamped", "moe_gated_experts", "headnorm_prepare", "channel_delta", "embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
        "paged_attention", "decode_attention_takes", "linear", "linear_swiglu", "tile_weight", "sample",
        "rmsnorm_addend", "gelu", "GELU_KINDS", "latent_prepare", "headwise_linear", "rotate_heads", "latent_attention",
        "moe_route", "moe_experts", "embed_streams", "hyper_norm", "causal_conv", "mamba2_scan", "gated_rmsnorm",
