@@ -29,10 +29,12 @@ class PreNormBlock(Part):
         super().__init__(prefix, precision, device)
         self.mixer = self.feed_forward = self.mixer_norm = self.feed_forward_norm = None
 
-    def attach(self, mixer, mixer_norm, feed_forward=None, feed_forward_norm=None):
+    def attach(self, mixer, feed_forward=None, mixer_norm=None, feed_forward_norm=None):
         """The layer's parts, under the names its LayerSpec gave them: a block's `attach` names
         the parts it arranges as its keywords, and a layer that brings others does not build. A
         layer without a feed-forward attaches the mixer and its norm only."""
+        if mixer_norm is None:
+            raise ValueError("a mixer comes with the norm before it")
         if (feed_forward is None) != (feed_forward_norm is None):
             raise ValueError("a feed-forward comes with its norm, or not at all")
         self.mixer = mixer

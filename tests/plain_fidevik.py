@@ -113,7 +113,7 @@ def choose_experts(z, correction, top, groups, keep):
 def routed_feed_forward(h, w, p, f):
     E, top = int(f["router"]["experts"]), int(f["router"]["top"])
     groups = f["router"].get("groups") or {"count": 1, "keep": 1}
-    z = h.to(torch.float32).to(h.dtype) @ w[p + ".router"].T
+    z = h @ w[p + ".router"].T
     chosen, share = choose_experts(z, w[p + ".correction"], top, int(groups["count"]), int(groups["keep"]))
     out = torch.zeros_like(h)
     for e in range(E):
