@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
                     [--shape 8b|14b|32b|0.6b] [--prompt P] [--context C]
-                    [--workload decode|continuous|served|prefix|products|kodisun|surasun|dufinex]
+                    [--workload decode|continuous|served|prefix|products|kodisun|surasun|dufinex|fidevik]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -693,6 +693,138 @@ def dufinex(args, sync):
     return 0
 
 
+FIDEVIK_SHAPES = {
+    # (width, query heads, key heads, q_rank, kv_rank, dense inner size, experts, top, groups, keep, expert_ff, shared_ff,
+    #  layers as (mixer, feed-forward), loop or None)
+    "base": (2048, 16, 4, 768, 512, 6144, 64, 6, 8, 4, 768, 1536,
+             (("attention", "dense"), ("latent_attention", "moe"), ("latent_attention", "moe"), ("attention", "moe")),
+             {"start": 1, "stop": 3, "times": 2}),
+    "wide": (4096, 32, 8, 1536, 512, 12288, 32, 4, 4, 2, 2048, 4096,
+             (("latent_attention", "moe"), ("attention", "dense")), None),
+}
+
+
+def fidevik(args, sync):
+    """Prefill and decode throughput of the Fidevik design at sizes that resemble a real model's layers
+    (random weights, a few layers, a vocabulary of 32,768), beside Kodisun, the closest of the other designs
+    (latent attention, a choice among small experts beside a shared one, a run of layers passed several
+    times), at the same width, head count, latent sizes, cached numbers per token, experts and run order,
+    with latent attention in every layer (64 of a head's 128 query numbers rotated) and the experts in
+    every layer. Both go through the engine's own loop: one prompt in one step, then greedy decoding at
+    batch 8 and 64 behind prompts of 1,024 tokens. `frac` prices a prompt's multiply-adds (the products
+    with a token's share of the experts, the attention's pairs in the form each design computes them)
+    against the bfloat16 matrix peak, and a decode step's bytes (the weights once, of the experts those a
+    batch can reach, the cached numbers its requests see) against the HBM peak."""
+    import torch
+
+    from qwen3_from_scratch_amd.config.fidevik_config import FidevikConfig
+    from qwen3_from_scratch_amd.config.kodisun_config import KodisunConfig
+    from qwen3_from_scratch_amd.engine import SyncEngine, random_model
+
+    vocab, prompt_len, decode_prompt, context = 32768, args.prefill_tokens, 1024, 4096
+    results = {}
+    for shape in ([args.fidevik_shape] if args.fidevik_shape != "all" else sorted(FIDEVIK_SHAPES)):
+        W, H, G, qr, kr, dense_ff, E, top, groups, keep, ff, sff, kinds, loop = FIDEVIK_SHAPES[shape]
+        if args.layers:
+            kinds, loop = (kinds * args.layers)[:args.layers], None
+        mixers = {"attention": {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                "rot": {"dims": 64, "base": 10000.0}},
+                  "latent_attention": {"heads": H, "dim": 128, "vdim": 128, "q_rank": qr, "kv_rank": kr, "scale": 128 ** -0.5}}
+        feeds = {"dense": {"kind": "dense", "ff": dense_ff},
+                 "moe": {"kind": "moe", "router": {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}},
+                         "expert": {"ff": ff}, "shared": {"ff": sff}}}
+        listed = [{"type": m, "mixer": mixers[m], "mlp": feeds[f]} for m, f in kinds]
+        data = {"architecture": "Fidevik", "vocab": vocab, "width": W, "norm": {"eps": 1e-5}, "logit_scale": 1.0, "layers": listed}
+        like = {"type": "latent_attention",
+                "mixer": {"heads": H, "dim": 64, "rot_dim": 64, "vdim": 128, "q_rank": qr, "kv_rank": kr - 64, "scale": 128 ** -0.5,
+                          "rot": {"dims": 64, "base": 10000.0}},
+                "mlp": {"kind": "moe", "router": {"experts": E, "top": top}, "expert": {"ff": ff}, "shared": {"ff": sff}}}
+        other = {"architecture": "Kodisun", "vocab": vocab, "width": W, "norm": {"eps": 1e-5}, "layers": [like] * len(kinds)}
+        if loop:
+            data["loop"] = other["loop"] = loop
+        for name, config in (("fidevik", FidevikConfig.from_dict(data)), ("kodisun", KodisunConfig.from_dict(other))):
+            if args.fidevik_only and name != args.fidevik_only:
+                continue
+            model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
+            gen = torch.Generator().manual_seed(1)
+            entry = {}
+            tensors = model.tensors()
+            # per run of a layer: matrix numbers every token meets, those of the experts (a token meets its share);
+            # multiply-adds per (query, key) pair in the form the design computes; numbers cached per token
+            matrices = expert_numbers = pairs_each = cached = 0
+            runs = [step.layer for step in model.spec.order]
+            for i in runs:
+                own = {key: t for key, t in tensors.items() if key.startswith("l%d." % i) and len(t) == 2}
+                expert_numbers += sum(t[0] * t[1] for key, t in own.items() if ".mlp.e" in key)
+                matrices += sum(t[0] * t[1] for key, t in own.items() if ".mlp.e" not in key)
+                layer = config.to_dict()["layers"][i]
+                m = layer["mixer"]
+                if layer["type"] == "attention":
+                    pairs_each += m["heads"] * (m["dim"] + m["vdim"])
+                    cached += m["kv_heads"] * (m["dim"] + m["vdim"])
+                else:                                    # in the latent's space: the cached row is key and value
+                    row = m["kv_rank"] + m.get("rot_dim", 0)
+                    pairs_each += m["heads"] * (row + m["kv_rank"])
+                    cached += row
+            share = top / E
+            if "prefill" in args.phases:
+                room = prompt_len + 64
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=room, block_size=BLOCK,
+                                    num_blocks=-(-room // BLOCK), max_num_seqs=1, max_num_tokens=prompt_len,
+                                    chunked_prefill_size=prompt_len, enable_prefix_cache=False)
+                timings = []
+                for _ in range(4):
+                    engine.add_request(torch.randint(0, vocab, (prompt_len,), generator=gen).tolist(),
+                                       engine.default_params(1, temperature=0.0, ignore_eos=True))
+                    sync()
+                    t0 = time.perf_counter()
+                    engine.step()
+                    sync()
+                    timings.append(time.perf_counter() - t0)
+                    while engine.scheduler.has_work():
+                        engine.step()
+                seconds = sorted(timings[1:])[1]
+                flops = (2.0 * prompt_len * (matrices + share * expert_numbers) + 2.0 * vocab * W
+                         + 2.0 * (prompt_len * (prompt_len + 1) / 2) * pairs_each)
+                entry["prefill"] = {"tokens": prompt_len, "tokens_per_s": round(prompt_len / seconds, 1),
+                                    "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+                del engine
+            for batch in ((8, 64) if "decode" in args.phases else ()):
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context,
+                                    block_size=BLOCK, num_blocks=batch * (context // BLOCK), max_num_seqs=batch,
+                                    max_num_tokens=max(2048, batch), chunked_prefill_size=2048, enable_prefix_cache=False)
+                params = engine.default_params(context - decode_prompt - 1, temperature=0.0, ignore_eos=True)
+                requests = [engine.add_request(torch.randint(0, vocab, (decode_prompt,), generator=gen).tolist(), params)
+                            for _ in range(batch)]
+                while any(r.is_prefill for r in requests) or len(engine.scheduler.waiting):
+                    engine.step()
+                for _ in range(args.warmup):
+                    engine.step()
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    engine.step()
+                sync()
+                step_s = (time.perf_counter() - t0) / args.steps
+                seen = decode_prompt + args.warmup + args.steps // 2
+                reached = min(1.0, batch * share)
+                # a layer's weights are read once per run of it: a pass finds little of the last pass's in the caches
+                need = 2 * (matrices + reached * expert_numbers + vocab * W) + batch * 2 * cached * seen
+                entry["decode_b%d" % batch] = {"tokens_per_s": round(batch / step_s, 1), "ms_per_step": round(step_s * 1e3, 3),
+                                               "frac_hbm": round(need / step_s / PEAK_HBM, 4)}
+                del engine
+            results.setdefault(shape, {})[name] = entry
+            del model
+            torch.cuda.empty_cache()
+        results[shape]["sizes"] = {"width": W, "heads": H, "kv_heads": G, "q_rank": qr, "kv_rank": kr, "dense_ff": dense_ff,
+                                   "experts": E, "top": top, "groups": groups, "keep": keep, "expert_ff": ff, "shared_ff": sff,
+                                   "vocab": vocab, "layers": ["%s+%s" % k for k in kinds], "loop": loop}
+    print(json.dumps({"metric": "Fidevik beside Kodisun at equal size: prefill and decode tokens/s",
+                      "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+                      "steps": args.steps, "warmup": args.warmup, "shapes": results}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -704,7 +836,7 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products", "kodisun", "surasun", "dufinex"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products", "kodisun", "surasun", "dufinex", "fidevik"],
                     help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
                          "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused); "
                          "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off; "
@@ -717,7 +849,10 @@ def main():
     ap.add_argument("--surasun-only", default="", choices=["", "surasun", "qwen3_dense"], help="one of the two models")
     ap.add_argument("--dufinex-shape", default="all", choices=["all"] + sorted(DUFINEX_SHAPES))
     ap.add_argument("--dufinex-only", default="", choices=["", "dufinex", "surasun"], help="one of the two models")
-    ap.add_argument("--phases", default="prefill,decode", help="of --workload kodisun, surasun or dufinex: prefill, decode or both")
+    ap.add_argument("--fidevik-shape", default="all", choices=["all"] + sorted(FIDEVIK_SHAPES))
+    ap.add_argument("--fidevik-only", default="", choices=["", "fidevik", "kodisun"], help="one of the two models")
+    ap.add_argument("--phases", default="prefill,decode",
+                    help="of --workload kodisun, surasun, dufinex or fidevik: prefill, decode or both")
     ap.add_argument("--single-copy", action="store_true",
                     help="hold the matrices once (no tile-ordered copy for steps of few rows): half the weights' memory, slower decoding")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
@@ -749,6 +884,10 @@ def main():
         torch.cuda.set_device(0)
         args.steps, args.warmup = min(args.steps, 32), min(args.warmup, 8)
         return dufinex(args, torch.cuda.synchronize)
+    if args.workload == "fidevik":
+        torch.cuda.set_device(0)
+        args.steps, args.warmup = min(args.steps, 32), min(args.warmup, 8)
+        return fidevik(args, torch.cuda.synchronize)
     shape_name, raw = SHAPES[args.shape]
     raw = dict(raw)
     prompt_len, context = args.prompt, args.context
