@@ -61,7 +61,9 @@ def fidevik_spec(config):
                          scale=config.logit_scale),
         pass_vectors=PartSpec.of("embedding", "pass_vectors", passes=times, hidden_size=width, leaf="step",
                                  restart=True) if looped else None,
-        pass_vectors_prefix="loop")
+        pass_vectors_prefix="loop",
+        # a loop over no layers at all still has its table of vectors in the file; nothing reads it
+        ignorable_tensors=() if looped else ("loop.step",))
 
 
 register_architecture(NAME, FidevikConfig, fidevik_spec)
