@@ -11,6 +11,17 @@ __device__ inline float moe_gelu(float z, int kind) {
   return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
 }
 
+// What the products' epilogues do with their sums (`act`): -1 nothing; 0, 1 the exact gelu and its tanh
+// form on every sum; from 2 on a gated unit over neighbouring columns, out[j] = g(sum[2j]) * sum[2j + 1]
+// with g silu (2), the tanh form of gelu (3) or the exact gelu (4): the weight's rows interleave gate
+// and up, the result has half the columns, and both sums enter unrounded.
+#define MOE_ACT_GATED 2
+#define MOE_ACT_MOST 4
+__device__ inline float moe_gated(float g, float u, int act) {
+  if (act == MOE_ACT_GATED) return g / (1.f + expf(-g)) * u;
+  return moe_gelu(g, act == 3 ? 1 : 0) * u;
+}
+
 // ---------------------------------------------------------------------------
 // The router's choice. One wavefront per token, from its float32 logits z (E numbers, a token's
 // `row_stride` apart). `mode` 0: s = softmax(z) over all E experts, then `top` times the largest
@@ -223,17 +234,25 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const T* __restrict__ x
 #pragma unroll
     for (int kk = 0; kk < MOE_BK; ++kk) {
       const float a = xs[r][kk];
+      // a gated unit wants a thread's four columns side by side; every sum's order over k is the same either way
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] += a * ws[c + 16 * j][kk];
+      for (int j = 0; j < 4; ++j) acc[j] += a * ws[act >= MOE_ACT_GATED ? 4 * c + j : c + 16 * j][kk];
     }
     __syncthreads();
   }
-  if (r < rows) {
+  if (r >= rows) return;
+  if (act >= MOE_ACT_GATED) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = n0 + c + 16 * j;
-      if (n < N) out[(size_t)(first + r) * N + n] = from_float<T>(act >= 0 ? moe_gelu(acc[j], act) : acc[j]);
+    for (int j = 0; j < 4; j += 2) {
+      const int n = n0 + 4 * c + j;
+      if (n + 1 < N) out[(size_t)(first + r) * (N / 2) + n / 2] = from_float<T>(moe_gated(acc[j], acc[j + 1], act));
     }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + c + 16 * j;
+    if (n < N) out[(size_t)(first + r) * N + n] = from_float<T>(act >= 0 ? moe_gelu(acc[j], act) : acc[j]);
   }
 }
 
@@ -329,6 +348,13 @@ __global__ __launch_bounds__(256) void moe_linear_mma_kernel(
 #pragma unroll
     for (int ns = 0; ns < NS; ++ns) {
       const int n = n_base + 16 * ns + 4 * grp;
+      if (act >= MOE_ACT_GATED) {                       // a lane's four columns are two (gate, up) pairs
+        bf16_t* o = out + (size_t)(first + m) * (N / 2) + n / 2;
+#pragma unroll
+        for (int i = 0; i < 4; i += 2)
+          if (n + i + 1 < N) o[i / 2] = float_to_bf16(moe_gated(acc[mt][ns][i], acc[mt][ns][i + 1], act));
+        continue;
+      }
       bf16_t* o = out + (size_t)(first + m) * N + n;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -447,6 +473,13 @@ __global__ __launch_bounds__(256) void moe_linear_big_kernel(
 #pragma unroll
     for (int ns = 0; ns < 2; ++ns) {
       const int n = n0 + 32 * wave + 16 * ns + 4 * grp;
+      if (act >= MOE_ACT_GATED) {
+        bf16_t* g = out + (size_t)(first + m) * (N / 2) + n / 2;
+#pragma unroll
+        for (int i = 0; i < 4; i += 2)
+          if (n + i + 1 < N) g[i / 2] = float_to_bf16(moe_gated(acc[mt][ns][i], acc[mt][ns][i + 1], act));
+        continue;
+      }
       bf16_t* o = out + (size_t)(first + m) * N + n;
       if (n + 3 < N && (N & 3) == 0) {
         union {
@@ -586,6 +619,13 @@ __global__ __launch_bounds__(64 * GT_WM * 2) void moe_linear_tiles_kernel(
       const int n = n0 + wn * (GT_BN / 2) + 16 * j + 4 * grp;
       if (n >= N) continue;
       f32x4_t c = acc[i][j];
+      if (act >= MOE_ACT_GATED) {
+        bf16_t* g = out + (size_t)(first_row + m) * (N / 2) + n / 2;
+#pragma unroll
+        for (int q = 0; q < 4; q += 2)
+          if (n + q + 1 < N) g[q / 2] = float_to_bf16(moe_gated(c[q], c[q + 1], act));
+        continue;
+      }
       if (act >= 0) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) c[q] = moe_gelu(c[q], act);
@@ -669,7 +709,8 @@ extern "C" int q3_moe_linear_mma(const void* x, const int* pair_of_slot, int gat
                                  void* out, const int* tile_expert, const int* tile_first, const int* offsets,
                                  const int* n_tiles, int max_tiles, int N, int K, int act, int tile_rows,
                                  hipStream_t stream) {
-  if (max_tiles <= 0 || N <= 0 || K <= 0 || K % 32 || pairs_per_row <= 0 || act < -1 || act > 1 ||
+  if (max_tiles <= 0 || N <= 0 || K <= 0 || K % 32 || pairs_per_row <= 0 || act < -1 || act > MOE_ACT_MOST ||
+      (act >= MOE_ACT_GATED && N % 2) ||
       (tile_rows != MMA_TM && tile_rows != BIG_TM && tile_rows != GT_BM))
     return Q3_ERR_BAD_ARGUMENT;
   if (tile_rows == GT_BM) {         // the dense path's copies and stages
@@ -713,7 +754,9 @@ extern "C" int q3_moe_linear(const void* x, const int* pair_of_slot, int gather,
                              void* out, const int* tile_expert, const int* tile_first, const int* offsets,
                              const int* n_tiles, int max_tiles, int N, int K, int act, int dtype,
                              hipStream_t stream) {
-  if (max_tiles <= 0 || N <= 0 || K <= 0 || pairs_per_row <= 0 || act < -1 || act > 1) return Q3_ERR_BAD_ARGUMENT;
+  if (max_tiles <= 0 || N <= 0 || K <= 0 || pairs_per_row <= 0 || act < -1 || act > MOE_ACT_MOST ||
+      (act >= MOE_ACT_GATED && N % 2))
+    return Q3_ERR_BAD_ARGUMENT;
   const dim3 grid(max_tiles, (N + MOE_BN - 1) / MOE_BN);
   if (grid.y > 65535) return Q3_ERR_UNSUPPORTED;
   Q3_DISPATCH_DTYPE(dtype, TT,

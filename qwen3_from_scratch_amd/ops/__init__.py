@@ -753,14 +753,17 @@ def moe_gated_experts(h, chosen, weights, gate_up, down, limit, slope):
     return out
 
 
+_MOE_ACT_GATED = 2      # the experts' product kernels: epilogue codes from here on are gated units, in the order of GATE_KINDS
+
+
 def moe_glu_experts(h, chosen, weights, gate_up, down, activation="silu", shared=None, shared_gate=None):
     """sum_k weights[t, k] * down[e] (act(gate[e] h[t]) * (up[e] h[t])), e = chosen[t, k]: experts that are
     gated units without biases, weighted on their results. h (T, width), gate_up (E, 2 ff, width) with rows
     2j the gate's and 2j + 1 the other branch's, down (E, width, ff), `activation` one of `GATE_KINDS`;
     `shared` (T, width) is added last, multiplied by sigmoid(shared_gate[t]) when `shared_gate` (float32
     (T,) or (T, 1), rows possibly apart: a logit per token) is given. Returns (T, width). The pairs are
-    sorted by expert on the GPU as in `moe_experts`; a token's sum is formed in float32 in the order of
-    its choices."""
+    sorted by expert on the GPU as in `moe_experts`; the gated unit is the epilogue of the first product,
+    from its float32 sums; a token's sum is formed in float32 in the order of its choices."""
     _dev(h, chosen, weights, gate_up, down, shared)
     T, width = h.shape
     E, ff = down.shape[0], down.shape[2]
@@ -785,16 +788,16 @@ def moe_glu_experts(h, chosen, weights, gate_up, down, activation="silu", shared
     many = 3 if width % 64 == 0 and ff % 64 == 0 else 2
     tile_rows = lib.q3_moe_tile_rows((many if P >= 96 * E else 1) if cores else 0)
     tiles, pair_of_slot, slot_of_pair = _moe_book(lib, chosen, E, tile_rows)
-    both = torch.empty((P, 2 * ff), dtype=h.dtype, device=h.device)
+    hidden = torch.empty((P, ff), dtype=h.dtype, device=h.device)
     y = torch.empty((P, width), dtype=h.dtype, device=h.device)
     stream = _stream()
+    gated = _MOE_ACT_GATED + GATE_KINDS[activation]      # the gated unit is the first product's epilogue, on unrounded sums
     if cores:
-        _check(lib.q3_moe_linear_mma(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(both), *tiles, 2 * ff, width,
-                                     -1, tile_rows, stream), "moe_linear")
+        _check(lib.q3_moe_linear_mma(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(hidden), *tiles, 2 * ff, width,
+                                     gated, tile_rows, stream), "moe_linear")
     else:
-        _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(both), *tiles, 2 * ff, width, -1,
-                                 _DT[h.dtype], stream), "moe_linear")
-    hidden = gated_act(both, activation)
+        _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(gate_up), _ptr(hidden), *tiles, 2 * ff, width,
+                                 gated, _DT[h.dtype], stream), "moe_linear")
     if cores:
         _check(lib.q3_moe_linear_mma(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff,
                                      -1, tile_rows, stream), "moe_linear")

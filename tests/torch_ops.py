@@ -375,8 +375,8 @@ def moe_glu_experts(h, chosen, weights, gate_up, down, activation="silu", shared
     out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
     for k in range(top):
         e = chosen[:, k].long()
-        both = torch.einsum("ti,tfi->tf", h.float(), gate_up[e].float()).to(h.dtype)
-        y = torch.einsum("tf,twf->tw", gated_act(both, activation).float(), down[e].float()).to(h.dtype)
+        both = torch.einsum("ti,tfi->tf", h.float(), gate_up[e].float())       # the gated unit sees unrounded sums
+        y = torch.einsum("tf,twf->tw", gated_act(both, activation).to(h.dtype).float(), down[e].float()).to(h.dtype)
         out += weights[:, k, None] * y.float()
     if shared is not None:
         out += shared.float() * (torch.sigmoid(shared_gate.reshape(T, 1)) if shared_gate is not None else 1.0)
