@@ -80,31 +80,18 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
       group_score[g] = size > 1 ? first + second : first;
     }
     __builtin_amdgcn_wave_barrier();
-    for (int k = 0; k < keep; ++k) {                        // the best group left, `keep` times; a kept group's score becomes NaN
-      float best = -INFINITY;
-      int at = 0x7fffffff;
-      for (int g = lane; g < groups; g += Q3_WAVE) {
-        const float p = group_score[g];
-        if (p > best || (at == 0x7fffffff && p == best)) {
-          best = p;
-          at = g;
-        }
+    // an expert stays if fewer than `keep` groups stand before its own (a higher score, or an equal one
+    // and a lower number): every lane ranks its expert's group against all of them, no round of maxima
+    for (int e = lane; e < E; e += Q3_WAVE) {
+      const int g = e / size;
+      const float own = group_score[g];
+      int before = 0;
+      for (int j = 0; j < groups; ++j) {
+        const float other = group_score[j];
+        before += (other > own || (other == own && j < g)) ? 1 : 0;
       }
-#pragma unroll
-      for (int off = Q3_WAVE / 2; off > 0; off >>= 1) {
-        const float ob = __shfl_xor(best, off, Q3_WAVE);
-        const int oa = __shfl_xor(at, off, Q3_WAVE);
-        if (ob > best || (ob == best && oa < at)) {
-          best = ob;
-          at = oa;
-        }
-      }
-      __builtin_amdgcn_wave_barrier();
-      if (at < groups) group_score[at] = NAN;
-      __builtin_amdgcn_wave_barrier();
+      if (before >= keep) z[e] = -INFINITY;
     }
-    for (int e = lane; e < E; e += Q3_WAVE)
-      if (group_score[e / size] == group_score[e / size]) z[e] = -INFINITY;      // not kept: still a number
     __builtin_amdgcn_wave_barrier();
   }
   const float nothing = mode == 0 ? -1.f : -INFINITY;     // below every score that can still be chosen
