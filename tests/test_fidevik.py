@@ -233,6 +233,23 @@ def test_run_order_and_cache_planes(cpu_ops, tmp_path):
     assert none.model.pass_vectors is None
 
 
+def test_a_loop_over_no_layers_is_no_loop(cpu_ops, tmp_path):
+    """start == stop: the layers run once, no pass begins, and the table of vectors that such a file may
+    still hold is left unread."""
+    data = dict(copy.deepcopy(STRAIGHT), loop={"start": 1, "stop": 1, "times": 2})
+    folder = _write(tmp_path / "m", data)
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    assert "loop.step" not in tensors
+    tensors["loop.step"] = torch.ones((2, data["width"]), dtype=torch.bfloat16)
+    save_file(tensors, path, metadata={"format": "pt"})
+    requests = {"a": random_tokens(20, data["vocab"], 3)}
+    _, _, want = _truth(folder, requests)
+    runner = load_runner(folder, dtype="float32", device="cpu", page_size=8, max_tokens=32, max_requests=1)
+    assert [(s.layer, s.enters) for s in runner.model.spec.order] == [(0, None), (1, None)]
+    assert _off(run_trace(runner, trace_whole(requests)), want, "float32") <= 1.0
+
+
 # ---- each mechanism alone, on the host twins and against the plain functions ----
 
 def test_layer_norm_twin_takes_every_addend(cpu_ops):
