@@ -33,4 +33,4 @@ class LinearHead(Part):
 
     def forward(self, h):
         logits = self.weight.forward(h, out_dtype=torch.float32)
-        return logits if self.scale == 1.0 else logits.mul_(self.scale)
+        return logits if self.scale == 1.0 else ops.scaled_sum(logits, self.scale, logits, 0.0)
